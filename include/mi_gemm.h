@@ -168,9 +168,11 @@ int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int ti
  * can show where a launch spends its time (per phase, per workgroup, per XCD).  Complements the whole-launch event
  * timing of the reference harness (gemm/gemm_test.cu:392-404), which has no in-kernel view.  Workgroup g writes
  * stamp i to d_stamps[(g * slots_per_workgroup + i) * 2] (the constant 100 MHz clock) and [... + 1] (the core clock
- * counter): stamp 0 at kernel entry, then for each work item of the workgroup one stamp at the end of its K loop and
- * one when its stores have been issued, and a last one when all stores have landed.  Stamps beyond
- * slots_per_workgroup are dropped.  The caller zero-fills d_stamps (2 * 8 bytes * slots * max_workgroups);
+ * counter): stamp 0 at kernel entry, then for each work item of the workgroup one stamp when its first K tile has
+ * landed in LDS, one at the end of its K loop and one when its stores have been issued, and a last one when all stores
+ * have landed.  The last slot is not a stamp: [0] = 1 + the wave's hardware id register (CU, shader array and shader
+ * engine in bits 8..15), [1] = the XCC (XCD) id, so that a tool can follow one CU through the launch.  Stamps beyond
+ * slots_per_workgroup - 1 are dropped.  The caller zero-fills d_stamps (2 * 8 bytes * slots * max_workgroups);
  * *out_workgroups receives the grid size; MI_ERR_WORKSPACE if that exceeds max_workgroups.  C is computed as usual. */
 int mi_matmul_mfma_timeline(const mi_gemm_tensors* t, int k_mode, int tile, uint64_t* d_stamps,
                             uint32_t slots_per_workgroup, uint32_t max_workgroups, uint32_t* out_workgroups,

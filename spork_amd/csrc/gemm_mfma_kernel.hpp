@@ -60,8 +60,9 @@ struct GemmArgs {
     // c + s * c_split_bytes with plain stores and a later pass sums the partitions.
     uint64_t c_split_bytes;
     // Diagnostic timeline (null in normal use): workgroup g writes stamp i to timeline[(g * timeline_slots + i) * 2]
-    // (the 100 MHz constant clock) and [.. + 1] (the core clock counter): kernel entry, then per work item the end of
-    // its K loop and the end of its epilogue issue, then the point where all of the workgroup's stores have landed.
+    // (the 100 MHz constant clock) and [.. + 1] (the core clock counter): kernel entry, then per work item the point where
+    // K tile 0 has landed, the end of its K loop and the end of its epilogue issue, then the point where all of the
+    // workgroup's stores have landed.  The last slot is not a stamp: it names the CU the workgroup ran on.
     unsigned long long* timeline;
     uint32_t timeline_slots;
 };
@@ -440,33 +441,49 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     AccT acc[MI][NI];
     u32x4 fa[2][MI], fb[2][NI];
 
-    // DMA instruction j of this wave: for j < A_DMA rows of A of K tile `tile_a` into the LDS region at byte `dst_a`,
-    // else rows of B of K tile `tile_b` into the region at `dst_b`
-    auto issue_dma = [&](auto jc, uint32_t tile_a, uint32_t tile_b, uint32_t dst_a, uint32_t dst_b) {
+    // Scalar byte offsets of the rows that DMA instruction jj of wave 0 fetches (the per-instruction part of the
+    // address): loop invariant, one SGPR each.
+    // ([0]: of the K tile the descriptor is based at, [1]: of the K tile after it)
+    uint32_t soff_a[2][A_DMA > 0 ? A_DMA : 1], soff_b[2][LPW - A_DMA > 0 ? LPW - A_DMA : 1];
+#pragma unroll
+    for (int jj = 0; jj < A_DMA; ++jj) {
+        soff_a[0][jj] = jj * a_jstride;
+        soff_a[1][jj] = jj * a_jstride + BK * 2;
+    }
+#pragma unroll
+    for (int jj = 0; jj < LPW - A_DMA; ++jj) {
+        soff_b[0][jj] = Cfg::template b_row<PERM>(jj) * ldb2;
+        soff_b[1][jj] = Cfg::template b_row<PERM>(jj) * ldb2 + BK * 2;
+    }
+    // DMA instruction j of this wave: for j < A_DMA rows of A into the LDS region at byte `dst_a`, else rows of B into
+    // the region at `dst_b`.  The K tile is the one the buffer descriptors `ka` / `kb` are based at (the first K
+    // element of some K tile of this item's panels), or the one after it (NEXT = 1): the descriptors advance by one
+    // K tile per iteration (two scalar adds) and the DMA itself needs no address arithmetic.  (The instruction's
+    // immediate offset cannot name the next K tile: an LDS DMA adds it to the LDS address as well.)
+    auto issue_dma = [&](auto jc, auto immc, const char* ka, const char* kb, uint32_t dst_a, uint32_t dst_b) {
         constexpr int j = jc.value;
+        constexpr int NEXT = immc.value;
         constexpr bool is_a = j < A_DMA;
         constexpr int jj = is_a ? j : j - A_DMA;
         const Item& it = cur;  // (captured by reference: the item lives for the whole kernel)
-        const uint32_t tile = is_a ? tile_a : tile_b;
-        const uint32_t koff = tile * (BK * 2);
         lds_char* const dst = lds_w + (is_a ? dst_a : dst_b) + jj * (NWAVES * 1024);
         if constexpr (!EDGE) {
             if constexpr (is_a) {
-                dma_buffer_to_lds_16B<ONCE == 1>(make_rsrc(it.a_base, BM * p.lda * 2u), voff_a, jj * a_jstride + koff, dst);
+                dma_buffer_to_lds_16B<ONCE == 1>(make_rsrc(ka, BM * p.lda * 2u), voff_a, soff_a[NEXT][jj], dst);
             }
             else {
-                dma_buffer_to_lds_16B<ONCE == 2>(make_rsrc(it.b_base, BN * p.ldb * 2u), voff_b, Cfg::template b_row<PERM>(jj) * ldb2 + koff,
-                                                 dst);
+                dma_buffer_to_lds_16B<ONCE == 2>(make_rsrc(kb, BN * p.ldb * 2u), voff_b, soff_b[NEXT][jj], dst);
             }
         }
         else {
             // the row part moves into the (range-checked) vector offset; a lane whose row or K chunk does not exist
             // asks for offset OOB instead
             const int32_t rows_left = is_a ? it.m_rem - jj * (NWAVES * RPI) : it.n_rem - (int32_t)Cfg::template b_row<PERM>(jj);
-            const int32_t k_left = it.k_rem - (int32_t)(tile * BK);
+            const int32_t k_done = (int32_t)((is_a ? ka - it.a_base : kb - it.b_base) / 2) + NEXT * BK;
+            const int32_t k_left = it.k_rem - k_done;
             const bool exists = (int32_t)(is_a ? lrow : lrow_b) < rows_left && (int32_t)(lchunk * 8u) < k_left;
             const uint32_t voff = (is_a ? voff_a + jj * a_jstride : voff_b + Cfg::template b_row<PERM>(jj) * ldb2);
-            dma_buffer_to_lds_16B(make_rsrc(is_a ? it.a_base : it.b_base, OOB), exists ? voff : OOB, koff, dst);
+            dma_buffer_to_lds_16B(make_rsrc(is_a ? ka : kb, OOB), exists ? voff : OOB, NEXT * (BK * 2), dst);
         }
     };
     // fragment read i of a k-step: B fragments first, then A fragments (the order the MFMA rows need them)
@@ -484,7 +501,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     uint32_t n_stamps = 0;
     auto stamp = [&]() {
         if (p.timeline != nullptr) {
-            if (threadIdx.x == 0 && n_stamps < p.timeline_slots) {
+            if (threadIdx.x == 0 && n_stamps + 1 < p.timeline_slots) {
                 unsigned long long* const dst = p.timeline + ((size_t)blockIdx.x * p.timeline_slots + n_stamps) * 2;
                 dst[0] = wall_clock64();
                 dst[1] = clock64();
@@ -533,10 +550,11 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
 #pragma unroll
         for (int t = 0; t < PF; ++t) {
             if ((uint32_t)t < cur.KT) {
-                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, t, t, ring_a(pos), ring_b(pos)); });
+                const char* const ka = cur.a_base + t * (BK * 2), * const kb = cur.b_base + t * (BK * 2);
+                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, ring_a(pos), ring_b(pos)); });
                 if (t < DIST_B) {
                     static_for<A_DMA, LPW>(
-                        [&](auto jc) { issue_dma(jc, t, t, ring_a(pos), ring_b(pos)); });
+                        [&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, ring_a(pos), ring_b(pos)); });
                 }
             }
             pos = ring_next(pos);
@@ -550,10 +568,8 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     else {
         wait_vmcnt_then_barrier<0>();
     }
+    stamp();
     static_for<0, NR>([&](auto ic) { issue_read(ic, IntC<0>{}, a_off[0], b_off[0] + ring_b(0)); });
-
-    uint32_t rd_pos = 0;                                          // ring position of tile kt
-    uint32_t pv_pos = SPLIT ? Cfg::UNITS - 2 : NSTAGE - 1;       // ring position of tile kt-1 (its refill may be in progress)
 
     {
         const uint32_t KT = cur.KT;
@@ -568,24 +584,38 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             }
         }
 
+        // Ring offsets in rotated order: u[k] is the LDS byte offset of ring position (position of tile kt) + k.  Moving
+        // on to the next K tile renames these scalars; no ring position is ever computed inside the loop.
+        constexpr int PERIOD = SPLIT ? Cfg::UNITS : NSTAGE;
+        constexpr int STEP = SPLIT ? 2 : 1;
+        uint32_t u[PERIOD];
+#pragma unroll
+        for (int k = 0; k < PERIOD; ++k) {
+            u[k] = (uint32_t)k * (SPLIT ? UNIT : (uint32_t)STAGE_BYTES);
+        }
+        // K tile kt + DIST - 1 of this item's panels (the rest of the refill begun in iteration kt-1 fetches it; the
+        // refill begun in iteration kt fetches the K tile after it, BK * 2 bytes on)
+        const char* ka = cur.a_base + (DIST_A - 1) * (BK * 2);
+        const char* kb = cur.b_base + (DIST_B - 1) * (BK * 2);
         // One K tile.  `steady` (compile time): every refill certainly happens, so the hot loop carries no branches;
         // otherwise (first and last PF iterations) they are decided at run time.
-        auto k_tile = [&](auto steady, uint32_t kt) {
+        auto k_tile = [&](auto steady, uint32_t kt) __attribute__((always_inline)) {
             constexpr bool STEADY = steady.value != 0;
-            const uint32_t nx_pos = ring_next(rd_pos);
-            const uint32_t a_cur = ring_a(rd_pos), b_cur = ring_b(rd_pos);
-            const uint32_t a_nxt = ring_a(nx_pos), b_nxt = ring_b(nx_pos);
+            // (split ring: the B tile sits in the unit after its A tile; slot ring: behind the A rows of the same slot)
+            constexpr int B_UNIT = SPLIT ? 1 : 0;
+            constexpr uint32_t B_BYTE = SPLIT ? 0u : (uint32_t)Cfg::A_BYTES;
+            const uint32_t a_cur = u[0], b_cur = u[B_UNIT] + B_BYTE;
+            const uint32_t a_nxt = u[STEP], b_nxt = u[STEP + B_UNIT] + B_BYTE;
             // Refill begun in this iteration, once tile kt has retired: A of tile kt+DIST_A and B of tile kt+DIST_B
             // into the regions tile kt occupied.
             const bool ra_on = STEADY || kt + DIST_A < KT, rb_on = STEADY || kt + DIST_B < KT;
-            const uint32_t ra_tile = kt + DIST_A, rb_tile = kt + DIST_B;
             const uint32_t ra_dst = SPLIT ? b_cur : a_cur, rb_dst = SPLIT ? a_cur : b_cur;
             // Rest of the refill begun in iteration kt-1 (its first part went out right after that tile's barrier).
             const bool pa_on = STEADY || (kt > 0 && kt + DIST_A < KT + 1);
             const bool pb_on = STEADY || (kt > 0 && kt + DIST_B < KT + 1);
-            const uint32_t pa_tile = kt + DIST_A - 1, pb_tile = kt + DIST_B - 1;
-            const uint32_t pa_dst = SPLIT ? ring_b(pv_pos) : ring_a(pv_pos);
-            const uint32_t pb_dst = SPLIT ? ring_a(pv_pos) : ring_b(pv_pos);
+            const uint32_t pv_a = u[PERIOD - STEP], pv_b = u[PERIOD - STEP + B_UNIT] + B_BYTE;
+            const uint32_t pa_dst = SPLIT ? pv_b : pv_a;
+            const uint32_t pb_dst = SPLIT ? pv_a : pv_b;
             static_for<0, KS>([&](auto ksc) {
                 constexpr int ks = ksc.value, cu = ks & 1, nx = cu ^ 1;
                 constexpr bool last = ks == KS - 1;
@@ -619,8 +649,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                 static_for<0, NI>([&](auto ni) { touch(fb[cu][ni.value]); });
                 touch(fa[cu][0]);
                 static_for<0, NMFMA>([&](auto ic) {
-                    constexpr int i = ic.value, mi = i / NI, ni = i % NI;
-                    if constexpr (ni == 0 && mi > 0) {
+                    // rows of MFMA tiles are walked boustrophedon: at a row change only the A operand changes (the
+                    // chip is power-limited and the operand buses toggle less: measured +0.5 % on 8192^3)
+                    constexpr int i = ic.value, mi = i / NI, ni_seq = i % NI, ni = (mi & 1) ? NI - 1 - ni_seq : ni_seq;
+                    if constexpr (ni_seq == 0 && mi > 0) {
                         if constexpr (!last) {
                             // outstanding: A fragments mi+1.. of this k-step, plus the reads issued so far for the next
                             // (the counter is 4 bits wide: a clamped wait is merely stricter)
@@ -641,12 +673,12 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                             constexpr int j = Cfg::dma_index(dma_lo + dc.value);
                             if constexpr (last) {
                                 if (j < A_DMA ? ra_on : rb_on) {
-                                    issue_dma(IntC<j>{}, ra_tile, rb_tile, ra_dst, rb_dst);
+                                    issue_dma(IntC<j>{}, IntC<1>{}, ka, kb, ra_dst, rb_dst);
                                 }
                             }
                             else {
                                 if (j < A_DMA ? pa_on : pb_on) {
-                                    issue_dma(IntC<j>{}, pa_tile, pb_tile, pa_dst, pb_dst);
+                                    issue_dma(IntC<j>{}, IntC<0>{}, ka, kb, pa_dst, pb_dst);
                                 }
                             }
                         }
@@ -655,8 +687,18 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                 });
                 static_for<Cfg::LOOP_READS, NR>([&](auto ic) { issue_read(ic, IntC<nx>{}, a_nx, b_nx); });
             });
-            pv_pos = rd_pos;
-            rd_pos = nx_pos;
+            // on to the next K tile: the ring turns by STEP positions
+            uint32_t turned[PERIOD];
+#pragma unroll
+            for (int k = 0; k < PERIOD; ++k) {
+                turned[k] = u[(k + STEP) % PERIOD];
+            }
+#pragma unroll
+            for (int k = 0; k < PERIOD; ++k) {
+                u[k] = turned[k];
+            }
+            ka += BK * 2;
+            kb += BK * 2;
         };
         {
             uint32_t kt = 0;
@@ -682,7 +724,17 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         const int32_t m_left = cur.m_rem - (int32_t)(wm * Cfg::TM) - (int32_t)(4u * g);  // rows from this lane's first row
         const int32_t n_left = cur.n_rem - (int32_t)(wn * Cfg::TN);  // columns from this wave's first column
         if constexpr (ATOMIC) {
-            float* cw = c_wave + (size_t)(4u * g) * p.ldc;
+            // Buffer atomics addressed like the plain stores below: a fixed per-lane 32-bit offset, the register-dependent
+            // rest a scalar offset, so the epilogue computes no per-element addresses.  One dword per lane, two full
+            // 128 B (MT = 32) or four 64 B (MT = 16) row segments per instruction.  Range-checked build: elements outside
+            // C get the out-of-range offset and the buffer range check drops the atomic.
+            const __amdgpu_buffer_rsrc_t rsrc_c = make_rsrc(c_wave, EDGE ? OOB : ((Cfg::TM - 1) * p.ldc + Cfg::TN) * 4u);
+            const uint32_t voff = (4u * g * p.ldc + lrc) * 4u;
+            // An atomic takes its data from an ordinary vector register.  Each value is moved out of its accumulation
+            // register right where it is used: left to itself the compiler moves all of them first and runs out of
+            // registers.  (The moves are opaque to the compiler's hazard pass, hence the explicit wait for the last
+            // MFMAs' results.)
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
@@ -690,14 +742,19 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
 #pragma unroll
                     for (int r = 0; r < NACC; ++r) {
                         const int row = mi * MT + row_of(r);
-                        const float v = acc[mi][ni][r];
-                        const uint32_t col = Cfg::template acc_col<PERM>(ni, lrc);
-                        if (!EDGE || (row < m_left && (int32_t)col < n_left)) {
-                            __hip_atomic_fetch_add(cw + (size_t)row * p.ldc + col, v, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
+                        const uint32_t soff = ((uint32_t)row * p.ldc + ni * MT) * 4u;
+                        float v;
+                        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[mi][ni][r]));
+                        if constexpr (!EDGE) {
+                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, rsrc_c, voff, soff, 0);
+                        }
+                        else {
+                            const bool inside = row < m_left && (int32_t)(ni * MT + lrc) < n_left;
+                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, rsrc_c, inside ? voff + soff : OOB, 0u, 0);
                         }
                     }
                 }
+                sched_fence();
             }
         }
         else {
@@ -799,6 +856,13 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         }
     }
     }  // parts
+    if (p.timeline != nullptr && threadIdx.x == 0 && p.timeline_slots > 0) {
+        // where this workgroup ran: the last slot holds 1 + the hardware id register (CU, shader array, shader engine) and
+        // the XCC id, so that a host tool can follow one CU through the launch
+        unsigned long long* const dst = p.timeline + ((size_t)blockIdx.x * p.timeline_slots + (p.timeline_slots - 1)) * 2;
+        dst[0] = 1ull + __builtin_amdgcn_s_getreg((31 << 11) | 4);
+        dst[1] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 15u;
+    }
 }
 
 }  // namespace mi_gemm

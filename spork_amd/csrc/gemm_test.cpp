@@ -272,11 +272,14 @@ int gemm_timeline(TimelineParams params, gpu_stream_t stream)
 
     auto wall = [&](uint32_t g, uint32_t i) { return h[(size_t(g) * SLOTS + i) * 2]; };
     auto core = [&](uint32_t g, uint32_t i) { return h[(size_t(g) * SLOTS + i) * 2 + 1]; };
+    // the last slot names the CU: hardware id register + 1 (CU, shader array, shader engine in bits 8..15) and XCC id
+    auto xcc_of = [&](uint32_t g) { return uint32_t(core(g, SLOTS - 1)); };
+    auto cu_key = [&](uint32_t g) { return xcc_of(g) << 8 | (uint32_t(wall(g, SLOTS - 1) - 1) >> 8 & 0xffu); };
     uint64_t t0 = ~uint64_t(0), t1 = 0;
     uint32_t max_stamps = 0;
     std::vector<uint32_t> count(wgs, 0);
     for (uint32_t g = 0; g < wgs; ++g) {
-        while (count[g] < SLOTS && wall(g, count[g]) != 0) {
+        while (count[g] < SLOTS - 1 && wall(g, count[g]) != 0) {
             ++count[g];
         }
         max_stamps = std::max(max_stamps, count[g]);
@@ -289,59 +292,114 @@ int gemm_timeline(TimelineParams params, gpu_stream_t stream)
     printf("timeline %ux%ux%u %s, tile %s, %s, %i K split(s): %u workgroups, up to %u stamps each\n", params.M, params.N,
            params.K, bf16 ? "bf16" : "f16", mi_tile_name(tile), mi_k_mode_name(k_mode), k_splits, wgs, max_stamps);
     printf("first entry to last store landed: %.2f us = %.1f TFLOP/s\n", span_us, 2.0 * M * N * K / span_us * 1e-6);
-    if (max_stamps < 3) {
+    if (max_stamps < 5) {
         printf("no stamps recorded\n");
         return 1;
     }
-    // phases: stamp 0 entry | per item: K loop end, stores issued | last: stores landed
-    printf("%-28s %10s %10s %10s %10s\n", "phase (us)", "min", "mean", "max", "core MHz");
-    for (uint32_t i = 1; i < max_stamps; ++i) {
+    struct Stat {
         double mn = 1e30, mx = 0, sum = 0, mhz = 0;
         uint32_t n = 0;
-        for (uint32_t g = 0; g < wgs; ++g) {
-            if (count[g] != max_stamps) {
-                continue;  // workgroups with fewer items are left out of the per-phase rows
-            }
-            const double us = double(wall(g, i) - wall(g, i - 1)) * 0.01;
+        void add(double us, double cycles)
+        {
             mn = std::min(mn, us);
             mx = std::max(mx, us);
             sum += us;
-            mhz += us > 0 ? double(core(g, i) - core(g, i - 1)) / us : 0;
+            mhz += us > 0 ? cycles / us : 0;
             ++n;
         }
-        if (n == 0) {
-            continue;
+        void print(const char* label) const
+        {
+            if (n) {
+                printf("%-34s %10.2f %10.2f %10.2f %10.0f %8u\n", label, mn, sum / n, mx, mhz / n, n);
+            }
+        }
+    };
+    // stamps: 0 entry | per item: K tile 0 landed, K loop end, stores issued | last: stores landed
+    static const char* const phase_name[3] = {"wait for K tile 0", "K loop", "store issue"};
+    printf("%-34s %10s %10s %10s %10s %8s\n", "phase (us)", "min", "mean", "max", "core MHz", "count");
+    for (uint32_t i = 1; i < max_stamps; ++i) {
+        Stat st;
+        for (uint32_t g = 0; g < wgs; ++g) {
+            if (count[g] == max_stamps) {  // workgroups with fewer items are left out of the per-phase rows
+                st.add(double(wall(g, i) - wall(g, i - 1)) * 0.01, double(core(g, i) - core(g, i - 1)));
+            }
         }
         char label[64];
         if (i + 1 == max_stamps) {
             snprintf(label, sizeof label, "stores landed");
         }
-        else if (i % 2 == 1) {
-            snprintf(label, sizeof label, "item %u K loop", (i - 1) / 2);
-        }
         else {
-            snprintf(label, sizeof label, "item %u store issue", (i - 1) / 2);
+            snprintf(label, sizeof label, "item %u %s", (i - 1) / 3, phase_name[(i - 1) % 3]);
         }
-        printf("%-28s %10.2f %10.2f %10.2f %10.0f\n", label, mn, sum / n, mx, mhz / n);
+        st.print(label);
     }
-    // workgroups are dealt round-robin to the 8 XCDs
-    printf("%-28s %10s %10s %10s\n", "workgroups end, by XCD (us)", "first", "last", "K-loop MHz");
-    for (uint32_t x = 0; x < 8 && x < wgs; ++x) {
+    // One CU through the launch: its workgroups in order of entry.  `turn` = how many workgroups the CU ran before.
+    std::vector<uint32_t> order(wgs);
+    for (uint32_t g = 0; g < wgs; ++g) {
+        order[g] = g;
+    }
+    std::sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
+        return cu_key(x) != cu_key(y) ? cu_key(x) < cu_key(y) : wall(x, 0) < wall(y, 0);
+    });
+    constexpr uint32_t TURNS = 8;
+    Stat gap_landed[TURNS], gap_issued[TURNS], fill[TURNS], loop[TURNS], store[TURNS], life[TURNS];
+    uint32_t cus_seen = 0, overlapped = 0;
+    for (uint32_t i = 0, turn = 0; i < wgs; ++i) {
+        const uint32_t g = order[i];
+        if (count[g] < 5) {
+            continue;
+        }
+        const bool same_cu = i > 0 && cu_key(order[i - 1]) == cu_key(g) && count[order[i - 1]] >= 5;
+        turn = same_cu ? turn + 1 : 0;
+        cus_seen += same_cu ? 0 : 1;
+        const uint32_t tr = std::min(turn, TURNS - 1);
+        if (same_cu) {
+            const uint32_t q = order[i - 1];
+            const double from_landed = (double(wall(g, 0)) - double(wall(q, count[q] - 1))) * 0.01;
+            const double from_issued = (double(wall(g, 0)) - double(wall(q, count[q] - 2))) * 0.01;
+            overlapped += from_issued < 0 ? 1 : 0;  // (two workgroups at once on the CU: tiles with a half-LDS ring)
+            gap_landed[tr].add(from_landed, 0);
+            gap_issued[tr].add(from_issued, 0);
+        }
+        fill[tr].add(double(wall(g, 1) - wall(g, 0)) * 0.01, double(core(g, 1) - core(g, 0)));
+        loop[tr].add(double(wall(g, 2) - wall(g, 1)) * 0.01, double(core(g, 2) - core(g, 1)));
+        store[tr].add(double(wall(g, 3) - wall(g, 2)) * 0.01, double(core(g, 3) - core(g, 2)));
+        life[tr].add(double(wall(g, count[g] - 1) - wall(g, 0)) * 0.01, double(core(g, count[g] - 1) - core(g, 0)));
+    }
+    printf("%u CUs seen; by the workgroup's turn on its CU (first item of each workgroup)%s\n", cus_seen,
+           overlapped ? "; workgroups overlap on a CU" : "");
+    for (uint32_t tr = 0; tr < TURNS; ++tr) {
+        char label[64];
+        snprintf(label, sizeof label, "turn %u%s: previous landed -> entry", tr, tr + 1 == TURNS ? "+" : "");
+        gap_landed[tr].print(label);
+        snprintf(label, sizeof label, "turn %u%s: previous issued -> entry", tr, tr + 1 == TURNS ? "+" : "");
+        gap_issued[tr].print(label);
+        snprintf(label, sizeof label, "turn %u%s: wait for K tile 0", tr, tr + 1 == TURNS ? "+" : "");
+        fill[tr].print(label);
+        snprintf(label, sizeof label, "turn %u%s: K loop", tr, tr + 1 == TURNS ? "+" : "");
+        loop[tr].print(label);
+        snprintf(label, sizeof label, "turn %u%s: store issue", tr, tr + 1 == TURNS ? "+" : "");
+        store[tr].print(label);
+        snprintf(label, sizeof label, "turn %u%s: entry -> landed", tr, tr + 1 == TURNS ? "+" : "");
+        life[tr].print(label);
+    }
+    printf("%-34s %10s %10s %10s %8s\n", "workgroups end, by XCD (us)", "first", "last", "K-loop MHz", "count");
+    for (uint32_t x = 0; x < 8; ++x) {
         double mn = 1e30, mx = 0, mhz = 0;
         uint32_t n = 0;
-        for (uint32_t g = x; g < wgs; g += 8) {
-            if (count[g] < 3) {
+        for (uint32_t g = 0; g < wgs; ++g) {
+            if (count[g] < 5 || xcc_of(g) != x) {
                 continue;
             }
             const double fin = double(wall(g, count[g] - 1) - t0) * 0.01;
             mn = std::min(mn, fin);
             mx = std::max(mx, fin);
-            const double us = double(wall(g, 1) - wall(g, 0)) * 0.01;  // first K loop of the workgroup
-            mhz += us > 0 ? double(core(g, 1) - core(g, 0)) / us : 0;
+            const double us = double(wall(g, 2) - wall(g, 1)) * 0.01;  // first K loop of the workgroup
+            mhz += us > 0 ? double(core(g, 2) - core(g, 1)) / us : 0;
             ++n;
         }
         if (n) {
-            printf("xcd %-24u %10.2f %10.2f %10.0f\n", x, mn, mx, mhz / n);
+            printf("xcd %-30u %10.2f %10.2f %10.0f %8u\n", x, mn, mx, mhz / n, n);
         }
     }
     fflush(stdout);

@@ -357,7 +357,7 @@ def test_mfma_auto_takes_the_workspace_sum_when_given_room(gpu, oracle):
                                         ((150, 77, 200), "TILE_AUTO")])
 def test_mfma_timeline_entry(gpu, oracle, shape, tile):
     """The diagnostic launch computes the same C and every workgroup leaves ordered stamps: entry, then per work item
-    the end of its K loop and of its store issue, then stores landed."""
+    K tile 0 landed, the end of its K loop and of its store issue, then stores landed; the last slot names the CU."""
     M, N, K = shape
     a, b = H.make_inputs(M, N, K, 1, 3, 3, 1.0, 0, 1)
     c = H.poisoned_c(M, N)
@@ -372,8 +372,9 @@ def test_mfma_timeline_entry(gpu, oracle, shape, tile):
     st = stamps.cpu().numpy()
     assert 1 <= wgs <= max_wg
     assert (st[wgs:] == 0).all()
-    n = (st[:wgs, :, 0] != 0).sum(axis=1)
-    assert (n >= 4).all() and (n % 2 == 0).all()      # entry + 2 per item + landed
+    assert (st[:wgs, slots - 1, 0] != 0).all() and (st[:wgs, slots - 1, 1] < 8).all()   # hardware id + 1, XCC id
+    n = (st[:wgs, :slots - 1, 0] != 0).sum(axis=1)
+    assert (n >= 5).all() and (n % 3 == 2).all()      # entry + 3 per item + landed
     for g in range(wgs):
         wall = st[g, :n[g], 0]
         core = st[g, :n[g], 1]
