@@ -140,6 +140,19 @@ int mi_matmul_mfma_workspace_bytes_for(const mi_gemm_tensors* t, int k_mode, int
 int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_workspace, size_t workspace_bytes,
                       void* hip_stream);
 
+/* mi_matmul_mfma_ws without the workspace argument, for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its callers
+ * bring a StreamWorkspace that allocates on demand, gemm/gpu_tensor.h:48-67).  The workspace is an array of
+ * MI_STATIC_SCRATCH_BYTES inside the library's own code object; the call allocates and frees nothing.  Everything
+ * mi_matmul_mfma_ws accepts is accepted as long as the re-packed operands fit (MI_ERR_WORKSPACE otherwise); K partitions
+ * are summed from copies of C in what is left of the array, or fall back to atomics.  Each GPU the library runs on holds
+ * its own copy of the array until the process ends.  All calls on one GPU share it: calls that overlap in time on one GPU
+ * (two streams, two threads) race and must be serialised by the caller; calls on one stream are ordered.  Nothing in the
+ * array needs clearing between calls (every byte a call reads was written by that call).  The array's address is looked
+ * up at mi_rt_set_device, else on the first call on a device: make that first call outside a graph capture. */
+#define MI_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream);
+
 /* `batches` independent problems of one shape in one launch: problem l reads a + l*a_batch_stride and
  * b + l*b_batch_stride (16-bit elements) and writes c + l*c_batch_stride (floats); a stride of 0 means densely packed
  * (M*K, N*K, M*N).  This is the leading `L` dimension of the reference's generated kernels,

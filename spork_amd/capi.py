@@ -14,6 +14,7 @@ _HEADER = os.path.join(os.path.dirname(_HERE), "include", "mi_gemm.h")
 F16, BF16, F32 = 0, 1, 2
 F32_BF16X1, F32_BF16X3 = 0, 1
 K_OUTPUT_STATIONARY, K_SPLIT, K_AUTO, K_SPLIT_REDUCE, K_STREAM = 0, 1, 2, 3, 4
+STATIC_SCRATCH_BYTES = 64 << 20  # MI_STATIC_SCRATCH_BYTES
 TILE_AUTO, TILE_256x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_192x256 = 0, 1, 2, 3, 4, 5
 TILE_224x256, TILE_160x256, TILE_224x128, TILE_160x128, TILE_256x192, TILE_192x192 = 6, 7, 8, 9, 10, 11
 TILE_192x128, TILE_96x128 = 12, 13
@@ -101,6 +102,7 @@ def lib() -> C.CDLL:
     sig("mi_matmul_mfma_workspace_bytes", i32, [tp, C.POINTER(sz)])
     sig("mi_matmul_mfma_workspace_bytes_for", i32, [tp, i32, i32, C.POINTER(sz), C.POINTER(sz)])
     sig("mi_matmul_mfma_ws", i32, [tp, i32, i32, vp, sz, vp])
+    sig("mi_matmul_mfma_static", i32, [tp, i32, i32, vp])
     sig("mi_matmul_mfma_timeline", i32, [tp, i32, i32, vp, u32, u32, C.POINTER(u32), vp])
     sig("mi_matmul_mfma_batched", i32, [tp, u32, C.c_uint64, C.c_uint64, C.c_uint64, i32, i32, vp])
     sig("mi_mfma_ceiling", i32, [vp, sz, i32, i32, u32, vp, vp, C.POINTER(u32), C.POINTER(C.c_double), vp])
@@ -178,6 +180,11 @@ def matmul_mfma_ws(t: GpuTensors, workspace_ptr: int, workspace_bytes: int, k_mo
                    stream: int = 0) -> None:
     """Any layout / any K: operands the kernel cannot read in place are re-packed into the caller's workspace."""
     check(lib().mi_matmul_mfma_ws(C.byref(t), k_mode, tile, workspace_ptr, workspace_bytes, stream), "mi_matmul_mfma_ws")
+
+
+def matmul_mfma_static(t: GpuTensors, k_mode: int = K_AUTO, tile: int = TILE_AUTO, stream: int = 0) -> None:
+    """matmul_mfma_ws on the library's own scratch array (STATIC_SCRATCH_BYTES): the call allocates nothing."""
+    check(lib().mi_matmul_mfma_static(C.byref(t), k_mode, tile, stream), "mi_matmul_mfma_static")
 
 
 def matmul_mfma_batched(t: GpuTensors, batches: int, a_batch_stride: int = 0, b_batch_stride: int = 0,

@@ -4,6 +4,7 @@
 #include "gemm_mfma_launch.hpp"
 
 #include <cstdio>
+#include <mutex>
 
 namespace mi_gemm {
 
@@ -893,6 +894,38 @@ static int check_modes(const mi_gemm_tensors* t, int k_mode, int tile)
     return MI_OK;
 }
 
+// Scratch memory of mi_matmul_mfma_static: a device array that is part of the library's code object, so the entry point
+// never allocates.  Every GPU the library runs on holds its own copy, at its own address, until the process ends.  In
+// host code `scratch` is only a handle for hipGetSymbolAddress; the address that kernels and copies may use is the one
+// that call returns, looked up once per device with that device current.
+constexpr size_t STATIC_SCRATCH_BYTES = MI_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+int resolve_static_scratch(void** out)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex guard;
+    static void* address[MAX_DEVICES] = {};
+    int dev = 0;
+    MI_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        return MI_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> lock(guard);
+    if (address[dev] == nullptr) {
+        void* ptr = nullptr;
+        MI_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr || (uintptr_t)ptr % 256) {
+            return MI_ERR_HIP;
+        }
+        address[dev] = ptr;
+    }
+    if (out != nullptr) {
+        *out = address[dev];
+    }
+    return MI_OK;
+}
+
 struct TimelineRequest {
     unsigned long long* d_stamps;
     uint32_t slots, max_workgroups;
@@ -1347,6 +1380,22 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
         return MI_ERR_WORKSPACE;
     }
     return run_mfma(t, k_mode, tile, d_workspace, d_workspace ? workspace_bytes : 0, hip_stream);
+}
+
+int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream)
+{
+    if (const int st = check_modes(t, k_mode, tile)) {
+        return st;
+    }
+    // what must fit: the re-packed operands (the K partitions' copies of C take what is left, or K splits by atomics)
+    if (prepare(*t).ws_bytes > STATIC_SCRATCH_BYTES) {
+        return MI_ERR_WORKSPACE;
+    }
+    void* ptr = nullptr;
+    if (const int st = resolve_static_scratch(&ptr)) {
+        return st;
+    }
+    return run_mfma(t, k_mode, tile, ptr, STATIC_SCRATCH_BYTES, hip_stream);
 }
 
 const char* mi_tile_name(int tile)

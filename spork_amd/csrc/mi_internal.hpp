@@ -31,6 +31,10 @@ inline hipStream_t as_stream(void* s)
 // Number of compute units of the current device (cached per device).
 int device_compute_units();
 
+// Address, on the current device, of the scratch array behind mi_matmul_mfma_static (looked up on the first call per
+// device; `out` may be null).  Allocates nothing.
+int resolve_static_scratch(void** out);
+
 // Basic validation shared by every GEMM entry point: non-null, non-zero, known dtype, flags are 0/1.
 int validate_tensors(const mi_gemm_tensors* t);
 

@@ -91,6 +91,9 @@ int mi_rt_device_count(int* count)
 int mi_rt_set_device(int device)
 {
     MI_HIP_TRY(hipSetDevice(device));
+    // the set-up call of a process that uses this device: look up the address of the library's scratch array here, so
+    // that mi_matmul_mfma_static finds it ready (it looks it up itself, and reports a failure, when this did not)
+    (void)resolve_static_scratch(nullptr);
     return MI_OK;
 }
 

@@ -308,6 +308,21 @@ def test_ceiling_probe_validates_its_arguments():
     assert lib.mi_mfma_ceiling(4100, 1 << 26, S.BF16, 16, 10, 4096, 8192, C.byref(n), C.byref(f), None) == 2   # alignment
 
 
+def test_static_entry_checks_arguments_and_size_before_touching_the_device():
+    """mi_matmul_mfma_static refuses bad modes and operands whose re-packed copies exceed its scratch array before it
+    makes any HIP call, so the refusals can be checked without a GPU."""
+    lib = S.lib()
+    assert S.STATIC_SCRATCH_BYTES == 64 << 20
+    header = open(os.path.join(os.path.dirname(S.lib_path()), "..", "..", "include", "mi_gemm.h")).read()
+    assert re.search(r"#define\s+MI_STATIC_SCRATCH_BYTES\s+\(\(size_t\)64 << 20\)", header)
+    assert lib.mi_matmul_mfma_static(None, S.K_AUTO, S.TILE_AUTO, None) == 2
+    assert lib.mi_matmul_mfma_static(C.byref(_t(256, 256, 256)), 9, S.TILE_AUTO, None) == 2
+    # a column-major 8192 x 8192 A re-packs into 128 MiB, a 4096 x 4096 one into 32 MiB + 32 MiB for row-major B: fits
+    t = _t(8192, 8192, 8192, S.BF16, a_col_major=1)
+    assert lib.mi_matmul_mfma_static(C.byref(t), S.K_AUTO, S.TILE_AUTO, None) == 3
+    assert S.matmul_mfma_workspace_bytes(_t(4096, 4096, 4096, S.BF16, a_col_major=1, b_col_major=0)) == 64 << 20
+
+
 def test_timeline_entry_validates_its_buffer():
     lib = S.lib()
     t = _t(256, 256, 256)
