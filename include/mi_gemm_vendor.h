@@ -28,6 +28,12 @@ int mi_vendor_matmul(const mi_gemm_tensors* t, void* d_workspace, size_t workspa
 
 int mi_vendor_last_status(void);
 
+/* The rule mi_vendor_matmul applies to what hipblasLtMatmulAlgoGetHeuristic returns before it keeps an algorithm: the
+ * result's own state must be success (MI_ERR_UNSUPPORTED otherwise) and the workspace the algorithm asks for must fit
+ * the bytes the caller gave (MI_ERR_WORKSPACE otherwise), since every later call runs the kept algorithm with the
+ * caller's pointer and size.  Pure host arithmetic; exported so that the rule can be checked without a device. */
+int mi_vendor_accepts_algorithm(int heuristic_state, size_t algorithm_workspace_bytes, size_t given_workspace_bytes);
+
 /* Which hipBLASLt this process is bound to: the file the dynamic linker resolved `hipblasLtMatmul` from, copied
  * into out (NUL-terminated, truncated to out_size).  A process that has loaded another copy of the library first
  * (PyTorch's wheel bundles its own, under the same soname) is bound to that copy, not to the one under /opt/rocm, and

@@ -31,6 +31,21 @@ struct Prepared {
     hipblasLtMatrixLayout_t first = nullptr, second = nullptr, out = nullptr;
     hipblasLtMatmulAlgo_t algo;
     bool first_is_b = false;  // which caller buffer is hipBLASLt's "A"
+
+    // (entries of the plan cache live until the process ends; a plan that is not kept is destroyed by its maker)
+    void destroy()
+    {
+        if (desc) {
+            hipblasLtMatmulDescDestroy(desc);
+        }
+        for (hipblasLtMatrixLayout_t l : {first, second, out}) {
+            if (l) {
+                hipblasLtMatrixLayoutDestroy(l);
+            }
+        }
+        desc = nullptr;
+        first = second = out = nullptr;
+    }
 };
 
 std::mutex g_mutex;
@@ -61,7 +76,19 @@ bool ensure_handle()
 // hipBLASLt is column-major.  A row-major R x C buffer is a column-major C x R matrix with leading dimension C.
 // Row-major C[M,N] is the column-major N x M product  B_op (N x K) * A_op (K x M);
 // column-major C[M,N] is the product                 A_op (M x K) * B_op (K x N).
+int fill_plan(const mi_gemm_tensors& t, size_t ws_bytes, Prepared& p);
+
+// Builds the plan for one problem; on any failure everything created so far is destroyed again.
 int prepare(const mi_gemm_tensors& t, size_t ws_bytes, Prepared& p)
+{
+    const int st = fill_plan(t, ws_bytes, p);
+    if (st != MI_OK) {
+        p.destroy();
+    }
+    return st;
+}
+
+int fill_plan(const mi_gemm_tensors& t, size_t ws_bytes, Prepared& p)
 {
     const hipDataType in_type = t.ab_dtype == MI_BF16 ? HIP_R_16BF : HIP_R_16F;
     LT_TRY(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
@@ -120,15 +147,22 @@ int prepare(const mi_gemm_tensors& t, size_t ws_bytes, Prepared& p)
     hipblasLtMatmulPreference_t pref = nullptr;
     LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
     const uint64_t max_ws = ws_bytes;
-    LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws)));
-    hipblasLtMatmulHeuristicResult_t result;
+    hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+    hipblasLtMatmulHeuristicResult_t result{};
     int found = 0;
-    const hipblasStatus_t st =
-        hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.first, p.second, p.out, p.out, pref, 1, &result, &found);
+    if (st == HIPBLAS_STATUS_SUCCESS) {
+        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.first, p.second, p.out, p.out, pref, 1, &result, &found);
+    }
     hipblasLtMatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || found < 1) {
         g_last_status = (int)st;
-        return MI_ERR_UNSUPPORTED;
+        return st != HIPBLAS_STATUS_SUCCESS ? MI_ERR_HIP : MI_ERR_UNSUPPORTED;
+    }
+    // The algorithm is run with the caller's workspace pointer and size on every later call: one that was not reported
+    // usable, or that wants more room than the caller has, must never be cached.
+    if (const int verdict = mi_vendor_accepts_algorithm((int)result.state, result.workspaceSize, ws_bytes)) {
+        g_last_status = (int)result.state;
+        return verdict;
     }
     p.algo = result.algo;
     return MI_OK;
@@ -170,6 +204,17 @@ int mi_vendor_version(void)
         return -1;
     }
     return version;
+}
+
+int mi_vendor_accepts_algorithm(int heuristic_state, size_t algorithm_workspace_bytes, size_t given_workspace_bytes)
+{
+    if (heuristic_state != (int)HIPBLAS_STATUS_SUCCESS) {
+        return MI_ERR_UNSUPPORTED;
+    }
+    if (algorithm_workspace_bytes > given_workspace_bytes) {
+        return MI_ERR_WORKSPACE;
+    }
+    return MI_OK;
 }
 
 int mi_vendor_last_status(void)

@@ -37,6 +37,8 @@ def lib() -> C.CDLL:
         L.mi_vendor_last_status.argtypes = []
         L.mi_vendor_matmul.restype = C.c_int
         L.mi_vendor_matmul.argtypes = [C.POINTER(GpuTensors), C.c_void_p, C.c_size_t, C.c_void_p]
+        L.mi_vendor_accepts_algorithm.restype = C.c_int
+        L.mi_vendor_accepts_algorithm.argtypes = [C.c_int, C.c_size_t, C.c_size_t]
         L.mi_vendor_library.restype = C.c_int
         L.mi_vendor_library.argtypes = [C.c_char_p, C.c_size_t]
         L.mi_vendor_version.restype = C.c_int

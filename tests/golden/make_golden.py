@@ -7,6 +7,11 @@ come from Python integers and from numpy / torch library routines, so they pin t
 pcg3d_vectors.json  the integer hash of gemm/gemm_test.cu:34-53 evaluated with Python big integers
 gemm_small.npz      48x40x80 fp16 and bf16 operands (raw bits) in all four A/B storage layouts and C = A B in fp64
                     from numpy.matmul on the numpy/torch-widened values
+random_style_vectors.json
+                    elements of the reference's sparse random style (gemm/gemm_test.cu:73-91) worked out by hand from
+                    the Python-integer hash: zeros, fourth powers (numpy float32 arithmetic in the reference's order of
+                    operations) and every 1-in-100000 spike of 1000 among the first 1024 x 1024 coordinates, with the
+                    fp16 / bf16 bit patterns from numpy / torch casts
 """
 import json
 import os
@@ -70,6 +75,32 @@ def main():
         out[f"{name}_c_f64"] = aw @ bw
         out[f"{name}_abs_c_f64"] = np.abs(aw) @ np.abs(bw)
     np.savez_compressed(os.path.join(HERE, "gemm_small.npz"), **out)
+
+    # gemm/gemm_test.cu:76-89: randbits = pcg3d(x, y, 20010106); 1000 if randbits % 100000 == 0; else 0 unless
+    # randbits % 4 == 0; else v = (pcg3d(x, y, 19980724) % 1000000) * 1e-6f in fp32, value (v * v) * (v * v)
+    def random_style(x, y):
+        randbits = pcg3d_python(x, y, 20010106)
+        if randbits % 100000 == 0:
+            return "spike", np.float32(1000.0)
+        if randbits % 4 != 0:
+            return "zero", np.float32(0.0)
+        v = np.float32(pcg3d_python(x, y, 19980724) % 1000000) * np.float32(1e-6)
+        return "fourth_power", (v * v) * (v * v)
+
+    picked, seen = [], {"spike": 0, "zero": 0, "fourth_power": 0}
+    for y in range(1024):
+        for x in range(1024):
+            kind, val = random_style(x, y)
+            want = 64 if kind == "spike" else 12
+            if seen[kind] < want and (kind == "spike" or (x * 7 + y * 13) % 97 == 0):
+                seen[kind] += 1
+                f16 = int(np.float32(val).astype(np.float16).view(np.uint16))
+                bf16 = int(torch.tensor(float(val), dtype=torch.float32).to(torch.bfloat16).view(torch.int16).item()) & 0xFFFF
+                picked.append({"x": x, "y": y, "kind": kind, "f32_bits": int(np.float32(val).view(np.uint32)),
+                               "f16_bits": f16, "bf16_bits": bf16})
+    assert seen["spike"] >= 4 and seen["zero"] == 12 and seen["fourth_power"] == 12, seen
+    with open(os.path.join(HERE, "random_style_vectors.json"), "w") as f:
+        json.dump(picked, f, indent=0)
 
 
 if __name__ == "__main__":

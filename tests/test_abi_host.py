@@ -32,8 +32,8 @@ def test_vendor_library_exports_its_header():
     from spork_amd import vendor as V
 
     names = V.exported_symbols()
-    assert names == ["mi_vendor_enabled", "mi_vendor_last_status", "mi_vendor_library", "mi_vendor_matmul",
-                     "mi_vendor_version"]
+    assert names == ["mi_vendor_accepts_algorithm", "mi_vendor_enabled", "mi_vendor_last_status", "mi_vendor_library",
+                     "mi_vendor_matmul", "mi_vendor_version"]
     out = subprocess.run(["nm", "-D", "--defined-only", V.lib_path()], capture_output=True, text=True, check=True).stdout
     for n in names:
         assert re.search(rf"\bT {n}\b", out), n
@@ -48,6 +48,12 @@ def test_vendor_library_exports_its_header():
     t = _t(64, 64, 64)
     assert lib.mi_vendor_matmul(C.byref(t), None, 0, None) == 3
     assert lib.mi_vendor_matmul(C.byref(t), 4096, (32 << 20) - 1, None) == 3
+    # an algorithm is kept only if the heuristic reported it usable and its workspace fits what the caller gave
+    assert lib.mi_vendor_accepts_algorithm(0, 0, 32 << 20) == 0
+    assert lib.mi_vendor_accepts_algorithm(0, 32 << 20, 32 << 20) == 0
+    assert lib.mi_vendor_accepts_algorithm(0, (32 << 20) + 1, 32 << 20) == 3      # wants more room than there is
+    assert lib.mi_vendor_accepts_algorithm(0, 128 << 20, 0) == 3
+    assert lib.mi_vendor_accepts_algorithm(7, 0, 128 << 20) == 1                  # heuristic state not success
     # the comparator names the hipBLASLt it is bound to (no device needed)
     assert lib.mi_vendor_library(None, 0) == 2
     path = V.library()

@@ -142,6 +142,28 @@ def test_reference_random_style_statistics(oracle):
     assert rest.max() <= 1.0
 
 
+def test_reference_random_style_hand_evaluated_elements(oracle):
+    """Elements of the sparse random style worked out from Python integers and numpy float32 arithmetic
+    (tests/golden/make_golden.py): zeros, fourth powers and every spike of 1000 in the first 1024 x 1024 coordinates.
+    A wrong modulus, a wrong seed or v^2 for v^4 changes these bits."""
+    vecs = json.load(open(os.path.join(GOLD, "random_style_vectors.json")))
+    kinds = {v["kind"] for v in vecs}
+    assert kinds == {"zero", "fourth_power", "spike"} and len(vecs) >= 28
+    plain = {d: oracle.fill(1024, 1024, oracle.RANDOM, False, d) for d in (oracle.F16, oracle.BF16)}
+    swapped = {d: oracle.fill(1024, 1024, oracle.RANDOM, True, d) for d in (oracle.F16, oracle.BF16)}
+    for v in vecs:
+        x, y = v["x"], v["y"]
+        f32 = np.float32(oracle.element(y, x, oracle.RANDOM, False, oracle.F16))
+        assert int(f32.view(np.uint32)) == v["f32_bits"], v
+        for d, key in ((oracle.F16, "f16_bits"), (oracle.BF16, "bf16_bits")):
+            assert int(plain[d][y, x]) == v[key], v        # x is the column
+            assert int(swapped[d][x, y]) == v[key], v      # transpose rule: x is the row
+    # the fixture holds every spike of that range: the oracle has no other
+    spikes = {(v["x"], v["y"]) for v in vecs if v["kind"] == "spike"}
+    ys, xs = np.nonzero(oracle.widen(plain[oracle.F16], oracle.F16) == 1000)
+    assert {(int(x), int(y)) for x, y in zip(xs, ys)} == spikes
+
+
 # ------------------------------------------------------------------------------------------------- GEMMs
 @pytest.mark.parametrize("name,dtype", [("f16", 0), ("bf16", 1)])
 @pytest.mark.parametrize("a_col", [0, 1])
