@@ -153,6 +153,14 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
 #define MI_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream);
 
+/* Sets up, once per device, what the first launch of a kernel would otherwise set up on the fly (the opt-in to more
+ * than 64 KB of dynamic LDS, gemm/gemm_sm80.cu:473-475; the reference does it under std::call_once,
+ * gemm/gemm_sm90.cu:1218-1219): every GEMM kernel that mi_matmul_mfma (workspace_bytes = 0) or mi_matmul_mfma_ws /
+ * mi_matmul_mfma_static (workspace_bytes = the size that call will be given) would launch for this problem, mode and tile.
+ * Launches nothing and touches no operand.  For callers that capture the call into a HIP graph without a warm-up call:
+ * a kernel's attributes cannot be set while its stream is capturing, so either call this first or make one eager call. */
+int mi_matmul_mfma_prepare(const mi_gemm_tensors* t, int k_mode, int tile, size_t workspace_bytes);
+
 /* `batches` independent problems of one shape in one launch: problem l reads a + l*a_batch_stride and
  * b + l*b_batch_stride (16-bit elements) and writes c + l*c_batch_stride (floats); a stride of 0 means densely packed
  * (M*K, N*K, M*N).  This is the leading `L` dimension of the reference's generated kernels,
@@ -219,7 +227,12 @@ int mi_matmul_mfma_describe(const mi_gemm_tensors* t, int k_mode, int tile, size
  * ranks plans by: measured per-K-step and per-workgroup times, not a promise).  Repacking passes are not included. */
 int mi_matmul_mfma_estimate_us(const mi_gemm_tensors* t, int k_mode, int tile, size_t workspace_bytes, double* out_us);
 
+/* The tile family as data, so that bindings, tests and drivers enumerate it instead of restating it: tile codes run from
+ * 1 to mi_tile_count() - 1 (0 is MI_TILE_AUTO); mi_tile_shape gives a tile's rows and columns, how many workgroups of it
+ * share a CU and whether it has a 32-deep twin (any out pointer may be NULL; MI_ERR_BAD_ARGUMENT for an unknown code). */
+int mi_tile_count(void);
 const char* mi_tile_name(int tile);
+int mi_tile_shape(int tile, uint32_t* out_bm, uint32_t* out_bn, int* out_workgroups_per_cu, int* out_has_32_deep_twin);
 const char* mi_k_mode_name(int k_mode);
 
 /* ------------------------------------------------------------------------------- harness device helpers */

@@ -17,20 +17,7 @@ from .capi import (  # noqa: F401
     K_SPLIT,
     K_SPLIT_REDUCE,
     K_STREAM,
-    TILE_128x128,
-    TILE_64x128,
-    TILE_192x256,
-    TILE_224x256,
-    TILE_160x256,
-    TILE_224x128,
-    TILE_160x128,
-    TILE_256x192,
-    TILE_192x192,
-    TILE_192x128,
-    TILE_96x128,
-    TILE_256x128,
-    TILE_256x256,
-    TILE_AUTO,
+    TILE_CODES,
     GpuTensors,
     MiGemmError,
     build,
@@ -50,6 +37,10 @@ from .capi import (  # noqa: F401
     matmul_mfma_workspace_bytes_for,
     matmul_mfma_ws,
     matmul_mfma_static,
+    matmul_mfma_prepare,
+    tile_count,
+    tile_shape,
+    tiles,
     STATIC_SCRATCH_BYTES,
     matmul_mfma_timeline,
     matmul_mfma_batched,
@@ -60,3 +51,6 @@ from .capi import (  # noqa: F401
     F32_BF16X3,
     status_string,
 )
+
+# TILE_AUTO, TILE_256x256, ...: one name per MI_TILE_* enumerator of include/mi_gemm.h
+globals().update(TILE_CODES)

@@ -15,9 +15,19 @@ F16, BF16, F32 = 0, 1, 2
 F32_BF16X1, F32_BF16X3 = 0, 1
 K_OUTPUT_STATIONARY, K_SPLIT, K_AUTO, K_SPLIT_REDUCE, K_STREAM = 0, 1, 2, 3, 4
 STATIC_SCRATCH_BYTES = 64 << 20  # MI_STATIC_SCRATCH_BYTES
-TILE_AUTO, TILE_256x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_192x256 = 0, 1, 2, 3, 4, 5
-TILE_224x256, TILE_160x256, TILE_224x128, TILE_160x128, TILE_256x192, TILE_192x192 = 6, 7, 8, 9, 10, 11
-TILE_192x128, TILE_96x128 = 12, 13
+
+
+def _tile_codes() -> dict:
+    """TILE_AUTO, TILE_256x256, ...: the MI_TILE_* enumerators as the header lists them (the header is the one place
+    that names the tiles of the ABI; their shapes come from the library, see tile_shape)."""
+    text = re.sub(r"/\*.*?\*/", "", open(_HEADER).read(), flags=re.S)
+    codes = {f"TILE_{m.group(1)}": int(m.group(2)) for m in re.finditer(r"\bMI_TILE_(AUTO|\d+x\d+)\s*=\s*(\d+)", text)}
+    assert codes.get("TILE_AUTO") == 0 and sorted(codes.values()) == list(range(len(codes))), codes
+    return codes
+
+
+TILE_CODES = _tile_codes()
+globals().update(TILE_CODES)
 DATA_RANDOM, DATA_IDENTITY, DATA_TILED_NUMBERS, DATA_UNIFORM, DATA_NORMAL = 0, 1, 2, 3, 4
 
 
@@ -109,6 +119,9 @@ def lib() -> C.CDLL:
     sig("mi_matmul_f32_workspace_bytes", i32, [tp, i32, C.POINTER(sz)])
     sig("mi_matmul_f32_ws", i32, [tp, i32, i32, i32, vp, sz, vp])
     sig("mi_tile_name", C.c_char_p, [i32])
+    sig("mi_tile_count", i32, [])
+    sig("mi_tile_shape", i32, [i32, C.POINTER(u32), C.POINTER(u32), ip, ip])
+    sig("mi_matmul_mfma_prepare", i32, [tp, i32, i32, sz])
     sig("mi_k_mode_name", C.c_char_p, [i32])
     sig("mi_init_test_data", i32, [vp, u32, u32, i32, i32, i32, C.c_double, u32, vp])
     sig("mi_compare_tensors", i32, [vp, vp, u32, u32, vp, vp])
@@ -180,6 +193,28 @@ def matmul_mfma_ws(t: GpuTensors, workspace_ptr: int, workspace_bytes: int, k_mo
                    stream: int = 0) -> None:
     """Any layout / any K: operands the kernel cannot read in place are re-packed into the caller's workspace."""
     check(lib().mi_matmul_mfma_ws(C.byref(t), k_mode, tile, workspace_ptr, workspace_bytes, stream), "mi_matmul_mfma_ws")
+
+
+def tile_count() -> int:
+    """Tile codes run from 1 to tile_count() - 1 (0 is TILE_AUTO)."""
+    return int(lib().mi_tile_count())
+
+
+def tile_shape(tile: int) -> dict:
+    bm, bn, per_cu, twin = C.c_uint32(), C.c_uint32(), C.c_int(), C.c_int()
+    check(lib().mi_tile_shape(tile, C.byref(bm), C.byref(bn), C.byref(per_cu), C.byref(twin)), "mi_tile_shape")
+    return {"code": tile, "name": lib().mi_tile_name(tile).decode(), "bm": bm.value, "bn": bn.value,
+            "workgroups_per_cu": per_cu.value, "has_32_deep_twin": bool(twin.value)}
+
+
+def tiles() -> list:
+    """Every tile of the family, as the library reports it."""
+    return [tile_shape(i) for i in range(1, tile_count())]
+
+
+def matmul_mfma_prepare(t: GpuTensors, k_mode: int = K_AUTO, tile: int = TILE_AUTO, workspace_bytes: int = 0) -> None:
+    """Sets the attributes of every kernel the call would launch (needed before a first call inside a graph capture)."""
+    check(lib().mi_matmul_mfma_prepare(C.byref(t), k_mode, tile, workspace_bytes), "mi_matmul_mfma_prepare")
 
 
 def matmul_mfma_static(t: GpuTensors, k_mode: int = K_AUTO, tile: int = TILE_AUTO, stream: int = 0) -> None:

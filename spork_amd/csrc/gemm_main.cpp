@@ -52,7 +52,7 @@ int main(int argc, char** argv)
     }
     if (argc > 1 && strcmp(argv[1], "--timeline") == 0) {
         if (argc < 5) {
-            fprintf(stderr, "usage: gemm --timeline M N K [f16|bf16] [tile code 0..13]\n");
+            fprintf(stderr, "usage: gemm --timeline M N K [f16|bf16] [tile code, 0 = auto]\n");
             return 2;
         }
         TimelineParams tp{};
@@ -66,7 +66,7 @@ int main(int argc, char** argv)
     }
 
     int failures = 0;
-    uint32_t keep_bits = ~0u;      // --versus times three algorithms only
+    uint64_t keep_bits = ~uint64_t(0);  // --versus times three algorithms only
     double* out_ms = nullptr;
 
     // data_style 0: all three reference styles; 1: tiled x identity; 2: identity x tiled; 3: reference random;
@@ -92,33 +92,9 @@ int main(int argc, char** argv)
             if (matmul_mi355_supports(t, MI_K_AUTO, MI_TILE_AUTO)) {
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_auto);
             }
-            if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, MI_TILE_256x256)) {
-                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_256x256);
-            }
-            if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, MI_TILE_256x128)) {
-                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_256x128);
-            }
-            if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, MI_TILE_128x128)) {
-                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_128x128);
-            }
-            if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, MI_TILE_64x128)) {
-                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_64x128);
-            }
-            if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, MI_TILE_192x256)) {
-                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_192x256);
-            }
-            const struct {
-                int tile;
-                AlgorithmCode code;
-            } in_between[] = {{MI_TILE_224x256, AlgorithmCode::mi355_224x256}, {MI_TILE_160x256, AlgorithmCode::mi355_160x256},
-                              {MI_TILE_224x128, AlgorithmCode::mi355_224x128}, {MI_TILE_160x128, AlgorithmCode::mi355_160x128},
-                              {MI_TILE_256x192, AlgorithmCode::mi355_256x192},
-                              {MI_TILE_192x192, AlgorithmCode::mi355_192x192},
-                              {MI_TILE_192x128, AlgorithmCode::mi355_192x128},
-                              {MI_TILE_96x128, AlgorithmCode::mi355_96x128}};
-            for (const auto& tc : in_between) {
-                if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, tc.tile)) {
-                    params.algorithm_code_bits |= algorithm_code_bit(tc.code);
+            for (int tile = 1; tile < mi_tile_count(); ++tile) {  // every tile of the family, forced
+                if (matmul_mi355_supports(t, MI_K_OUTPUT_STATIONARY, tile)) {
+                    params.algorithm_code_bits |= algorithm_code_bit(forced_tile_algorithm(tile));
                 }
             }
             if (matmul_mi355_supports(t, MI_K_SPLIT, MI_TILE_AUTO)) {
@@ -254,7 +230,7 @@ int main(int argc, char** argv)
         }
         keep_bits = algorithm_code_bit(AlgorithmCode::mi355_auto) | algorithm_code_bit(AlgorithmCode::mi355_auto_ws) |
                     algorithm_code_bit(AlgorithmCode::hipblaslt);
-        double ms[64][algorithm_count] = {};
+        static double ms[64][algorithm_max_count] = {};
         for (uint32_t i = 0; i < shape_count; ++i) {
             out_ms = ms[i];
             sized_tests(shapes[i].M, shapes[i].N, shapes[i].K, 5, MI_BF16);

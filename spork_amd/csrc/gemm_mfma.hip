@@ -8,24 +8,39 @@
 
 namespace mi_gemm {
 
-MI_GEMM_DECLARE_CFG(Cfg256x256)
-MI_GEMM_DECLARE_CFG(Cfg256x128)
-MI_GEMM_DECLARE_CFG(Cfg128x128)
-MI_GEMM_DECLARE_CFG(Cfg64x128)
-MI_GEMM_DECLARE_CFG(Cfg256x256k32)
-MI_GEMM_DECLARE_CFG(Cfg256x128k32)
-MI_GEMM_DECLARE_CFG(Cfg128x128k32)
-MI_GEMM_DECLARE_CFG(Cfg64x128k32)
-MI_GEMM_DECLARE_CFG(Cfg192x256)
-MI_GEMM_DECLARE_CFG(Cfg192x256k32)
-MI_GEMM_DECLARE_CFG(Cfg224x256)
-MI_GEMM_DECLARE_CFG(Cfg160x256)
-MI_GEMM_DECLARE_CFG(Cfg224x128)
-MI_GEMM_DECLARE_CFG(Cfg160x128)
-MI_GEMM_DECLARE_CFG(Cfg256x192)
-MI_GEMM_DECLARE_CFG(Cfg192x192)
-MI_GEMM_DECLARE_CFG(Cfg192x128)
-MI_GEMM_DECLARE_CFG(Cfg96x128)
+#define MI_ROW_DECLARE(code, name, Cfg, ...) MI_GEMM_DECLARE_CFG(Cfg)
+MI_TILE_TABLE(MI_ROW_DECLARE)
+MI_TILE_TWINS(MI_GEMM_DECLARE_CFG)
+#undef MI_ROW_DECLARE
+
+// The tile family, indexed by ABI code - 1 (code 0 is MI_TILE_AUTO).
+#define MI_ROW_ENTRY(code, name, Cfg, Twin, us_k64, fixed_us, short_us, per_cu, alone_k64, alone_us, max_k) \
+    TileRow{code,                                                                                           \
+            name,                                                                                           \
+            Cfg::BM,                                                                                        \
+            Cfg::BN,                                                                                        \
+            {Launchers<Cfg>::f16, Launchers<Cfg>::bf16},                                                    \
+            {Launchers<Twin>::f16, Launchers<Twin>::bf16},                                                  \
+            us_k64,                                                                                         \
+            fixed_us,                                                                                       \
+            short_us,                                                                                       \
+            per_cu,                                                                                         \
+            alone_k64,                                                                                      \
+            alone_us,                                                                                       \
+            max_k},
+static const TileRow TILES[] = {MI_TILE_TABLE(MI_ROW_ENTRY)};
+#undef MI_ROW_ENTRY
+constexpr int TILE_ROWS = sizeof(TILES) / sizeof(TILES[0]);
+static_assert(TILE_ROWS == MI_TILE_COUNT_ - 1, "one table row per tile code of the ABI");
+
+// The row of a tile code, or null (MI_TILE_AUTO and unknown codes have none).
+static const TileRow* tile_row(int tile)
+{
+    if (tile < 1 || tile > TILE_ROWS || TILES[tile - 1].code != tile) {
+        return nullptr;
+    }
+    return &TILES[tile - 1];
+}
 
 struct TileDims {
     uint32_t bm, bn, bk;
@@ -43,23 +58,12 @@ static uint32_t slot_depth(uint32_t K)
 
 static bool tile_dims(int tile, uint32_t K, TileDims& d)
 {
-    switch (tile) {
-    case MI_TILE_256x256: d = {256, 256, slot_depth(K)}; return true;
-    case MI_TILE_256x128: d = {256, 128, slot_depth(K)}; return true;
-    case MI_TILE_128x128: d = {128, 128, slot_depth(K)}; return true;
-    case MI_TILE_64x128: d = {64, 128, slot_depth(K)}; return true;
-    case MI_TILE_192x256: d = {192, 256, slot_depth(K)}; return true;
-    // (no 32-deep twins: a K that is only a multiple of 32 runs their range-checked build with a half-empty last slot)
-    case MI_TILE_224x256: d = {224, 256, 64}; return true;
-    case MI_TILE_160x256: d = {160, 256, 64}; return true;
-    case MI_TILE_224x128: d = {224, 128, 64}; return true;
-    case MI_TILE_160x128: d = {160, 128, 64}; return true;
-    case MI_TILE_256x192: d = {256, 192, 64}; return true;
-    case MI_TILE_192x192: d = {192, 192, 64}; return true;
-    case MI_TILE_192x128: d = {192, 128, 64}; return true;
-    case MI_TILE_96x128: d = {96, 128, 64}; return true;
+    const TileRow* const row = tile_row(tile);
+    if (row == nullptr) {
+        return false;
     }
-    return false;
+    d = {row->bm, row->bn, row->twin[0] != nullptr ? slot_depth(K) : 64u};
+    return true;
 }
 
 static uint32_t ceil_div(uint32_t a, uint32_t b)
@@ -121,10 +125,11 @@ static Prepared prepare(const mi_gemm_tensors& t)
 }
 
 // Limits that hold whatever the tile: a 256-row panel must stay below the 2 GiB reach of a buffer descriptor's
-// 32-bit offsets, and C must be dword aligned.
+// 32-bit offsets, C must be dword aligned, and the range-checked build counts the rows that are left in 32-bit
+// signed integers.  (For a column-major C the canonical M is the caller's N: both sides are covered.)
 static bool problem_fits(const Canonical& c)
 {
-    return (uintptr_t)c.c % 4 == 0 && c.K < (1u << 21) && c.N < (1u << 21);
+    return (uintptr_t)c.c % 4 == 0 && c.K < (1u << 21) && c.N < (1u << 21) && c.M < (1u << 31);
 }
 
 static bool tile_fits(const Canonical& c, int tile, uint32_t k_splits)
@@ -217,22 +222,9 @@ static double stream_k_cost(const Canonical& c, int tile, uint32_t workgroups)
 {
     TileDims d;
     tile_dims(tile, c.K, d);
-    double us_per_k64 = 0.0, fixed_us = 0.0;
-    switch (tile) {
-    case MI_TILE_256x256: us_per_k64 = 1.33; fixed_us = 15.0; break;
-    case MI_TILE_256x128: us_per_k64 = 0.73; fixed_us = 10.0; break;
-    case MI_TILE_128x128: us_per_k64 = 0.44; fixed_us = 7.0; break;
-    case MI_TILE_64x128: us_per_k64 = 0.25; fixed_us = 6.0; break;
-    case MI_TILE_192x256: us_per_k64 = 1.03; fixed_us = 13.0; break;
-    case MI_TILE_224x256: us_per_k64 = 1.16; fixed_us = 13.5; break;
-    case MI_TILE_160x256: us_per_k64 = 0.86; fixed_us = 12.0; break;
-    case MI_TILE_224x128: us_per_k64 = 0.64; fixed_us = 9.5; break;
-    case MI_TILE_160x128: us_per_k64 = 0.48; fixed_us = 8.5; break;
-    case MI_TILE_256x192: us_per_k64 = 1.02; fixed_us = 13.0; break;
-    case MI_TILE_192x192: us_per_k64 = 0.755; fixed_us = 18.5; break;
-    case MI_TILE_192x128: us_per_k64 = 0.85; fixed_us = 12.0; break;  // (one workgroup per CU here)
-    case MI_TILE_96x128: us_per_k64 = 0.36; fixed_us = 6.5; break;
-    }
+    // (one workgroup per CU here)
+    const TileRow& row = *tile_row(tile);
+    const double us_per_k64 = row.alone_k64, fixed_us = row.alone_us;
     const double tiles = (double)(c.M / d.bm) * (c.N / d.bn), k_tiles = c.K / 64;
     const double run = __builtin_ceil(tiles * k_tiles / workgroups);
     const double tile_bytes = 4.0 * d.bm * d.bn, c_bytes = 4.0 * c.M * c.N;
@@ -254,30 +246,11 @@ static double plan_cost(const Canonical& c, int tile, uint32_t k_splits, bool re
 {
     TileDims d;
     tile_dims(tile, c.K, d);
-    double us_per_k64 = 0.0, fixed_us = 0.0;
-    double places = cus;  // workgroups that run side by side in one round
-    switch (tile) {
-    case MI_TILE_256x256: us_per_k64 = 1.33; fixed_us = 15.0; break;
-    case MI_TILE_256x128: us_per_k64 = 0.73; fixed_us = 10.0; break;
-    case MI_TILE_128x128: us_per_k64 = 0.44; fixed_us = 7.0; break;
-    case MI_TILE_64x128: us_per_k64 = 0.25; fixed_us = 6.0; break;
-    case MI_TILE_192x256: us_per_k64 = 1.03; fixed_us = 13.0; break;
-    case MI_TILE_224x256: us_per_k64 = 1.16; fixed_us = 13.5; break;
-    case MI_TILE_160x256: us_per_k64 = 0.86; fixed_us = 12.0; break;
-    case MI_TILE_224x128: us_per_k64 = 0.64; fixed_us = 9.5; break;
-    case MI_TILE_160x128: us_per_k64 = 0.48; fixed_us = 8.5; break;
-    case MI_TILE_256x192: us_per_k64 = 1.02; fixed_us = 13.0; break;
-    case MI_TILE_192x192: us_per_k64 = 0.755; fixed_us = 18.5; break;
-    case MI_TILE_192x128:
-        // Two workgroups share a CU (the ring is half of the LDS): a round has two places per CU, and these are the
-        // times of such a pair, measured on 7072 x 7352 x 1024, 6144 x 4096 x 1024, 8192^2 x 2048 and 8192^2 x 256
-        // (126, 53, 246, 65 us).  A CU that holds one alone takes 0.85 us per K step.
-        us_per_k64 = 1.0;
-        fixed_us = 9.0;
-        places = 2.0 * cus;
-        break;
-    case MI_TILE_96x128: us_per_k64 = 0.36; fixed_us = 6.5; break;
-    }
+    // (two workgroups share a CU when the ring is half of the LDS: a round then has two places per CU and the table
+    // holds the times of such a pair; a CU that holds one alone runs at alone_k64)
+    const TileRow& row = *tile_row(tile);
+    double us_per_k64 = row.us_k64, fixed_us = row.fixed_us;
+    const double places = (double)row.per_cu * cus;  // workgroups that run side by side in one round
     if (d.bk == 32) {
         us_per_k64 *= 1.1;  // half-line L2 requests and twice the barriers
     }
@@ -303,21 +276,7 @@ static double plan_cost(const Canonical& c, int tile, uint32_t k_splits, bool re
         // Measured per-workgroup cost on 8192 x 8192 x 64..384, 16384 x 16384 x 128 and 32768 x 65536 x 48: the
         // 256 x 256 tile's store burst is overlapped by nothing, smaller tiles interleave stores and loads across
         // the CUs, and rounds blur into each other.
-        switch (tile) {
-        case MI_TILE_256x256: fixed_us = 17.4; break;
-        case MI_TILE_192x256: fixed_us = 8.5; break;
-        case MI_TILE_256x128: fixed_us = 7.2; break;
-        case MI_TILE_128x128: fixed_us = 3.0; break;
-        case MI_TILE_64x128: fixed_us = 2.8; break;
-        case MI_TILE_224x256: fixed_us = 13.0; break;
-        case MI_TILE_160x256: fixed_us = 7.5; break;
-        case MI_TILE_224x128: fixed_us = 6.5; break;
-        case MI_TILE_160x128: fixed_us = 4.0; break;
-        case MI_TILE_256x192: fixed_us = 10.0; break;
-        case MI_TILE_192x192: fixed_us = 8.0; break;
-        case MI_TILE_192x128: fixed_us = 8.0; break;
-        case MI_TILE_96x128: fixed_us = 2.9; break;
-        }
+        fixed_us = row.short_us;
         waves = items / places;
     }
     else if (places == cus && waves > 4.0) {
@@ -447,12 +406,13 @@ static bool make_plan(const Canonical& c, int k_mode, int tile, size_t partial_s
 // and 2048, 3000 x 11008 x 4096 253 us against 214 us).
 static bool planner_considers(int tile, uint32_t K)
 {
-    return tile != MI_TILE_192x128 || K <= 1536;
+    const TileRow* const row = tile_row(tile);
+    return row != nullptr && (row->max_k == 0 || K <= row->max_k);
 }
 
 static bool search_plan(const Canonical& c, int k_mode, int tile, size_t partial_space, int cus, Plan& plan)
 {
-    const int tile_lo = tile == MI_TILE_AUTO ? MI_TILE_256x256 : tile;
+    const int tile_lo = tile == MI_TILE_AUTO ? 1 : tile;
     const int tile_hi = tile == MI_TILE_AUTO ? MI_TILE_COUNT_ - 1 : tile;
     bool found = false;
     double best = 0.0;
@@ -592,7 +552,7 @@ static Peel plan_peeled(const Canonical& c, int cus, double whole_cost_us)
     if (memo.valid && memo.M == c.M && memo.N == c.N && memo.K == c.K && memo.cus == cus && memo.whole_cost_us == whole_cost_us) {
         return memo.peel;
     }
-    for (int tl = MI_TILE_256x256; tl < MI_TILE_COUNT_; ++tl) {
+    for (int tl = 1; tl < MI_TILE_COUNT_; ++tl) {
         TileDims d;
         if (!tile_dims(tl, c.K, d) || !planner_considers(tl, c.K)) {
             continue;
@@ -762,42 +722,17 @@ static int stream_k_sum(const float* parts, const Canonical& c, const Plan& plan
     return MI_OK;
 }
 
-template <int DTYPE>
-static int launch_tile(const Canonical& problem, const Plan& plan, hipStream_t stream)
+static int launch_tile(int dtype, const Canonical& problem, const Plan& plan, hipStream_t stream)
 {
     TileDims d;
-    if (!tile_dims(plan.tile, problem.K, d)) {
+    const TileRow* const row = tile_row(plan.tile);
+    if (row == nullptr || !tile_dims(plan.tile, problem.K, d) || (dtype != MI_F16 && dtype != MI_BF16)) {
         return MI_ERR_BAD_ARGUMENT;
     }
     Canonical c = problem;
     c.read_once = problem.stream_k_workgroups ? 0 : read_once_operand(c, plan);
-    const bool deep = d.bk == 64, edge = needs_edge(c, d);
-    switch (plan.tile) {
-    case MI_TILE_256x256:
-        return deep ? launch_cfg<DTYPE, Cfg256x256>(c, plan.k_splits, edge, stream)
-                    : launch_cfg<DTYPE, Cfg256x256k32>(c, plan.k_splits, edge, stream);
-    case MI_TILE_256x128:
-        return deep ? launch_cfg<DTYPE, Cfg256x128>(c, plan.k_splits, edge, stream)
-                    : launch_cfg<DTYPE, Cfg256x128k32>(c, plan.k_splits, edge, stream);
-    case MI_TILE_128x128:
-        return deep ? launch_cfg<DTYPE, Cfg128x128>(c, plan.k_splits, edge, stream)
-                    : launch_cfg<DTYPE, Cfg128x128k32>(c, plan.k_splits, edge, stream);
-    case MI_TILE_64x128:
-        return deep ? launch_cfg<DTYPE, Cfg64x128>(c, plan.k_splits, edge, stream)
-                    : launch_cfg<DTYPE, Cfg64x128k32>(c, plan.k_splits, edge, stream);
-    case MI_TILE_192x256:
-        return deep ? launch_cfg<DTYPE, Cfg192x256>(c, plan.k_splits, edge, stream)
-                    : launch_cfg<DTYPE, Cfg192x256k32>(c, plan.k_splits, edge, stream);
-    case MI_TILE_224x256: return launch_cfg<DTYPE, Cfg224x256>(c, plan.k_splits, edge, stream);
-    case MI_TILE_160x256: return launch_cfg<DTYPE, Cfg160x256>(c, plan.k_splits, edge, stream);
-    case MI_TILE_224x128: return launch_cfg<DTYPE, Cfg224x128>(c, plan.k_splits, edge, stream);
-    case MI_TILE_160x128: return launch_cfg<DTYPE, Cfg160x128>(c, plan.k_splits, edge, stream);
-    case MI_TILE_256x192: return launch_cfg<DTYPE, Cfg256x192>(c, plan.k_splits, edge, stream);
-    case MI_TILE_192x192: return launch_cfg<DTYPE, Cfg192x192>(c, plan.k_splits, edge, stream);
-    case MI_TILE_192x128: return launch_cfg<DTYPE, Cfg192x128>(c, plan.k_splits, edge, stream);
-    case MI_TILE_96x128: return launch_cfg<DTYPE, Cfg96x128>(c, plan.k_splits, edge, stream);
-    }
-    return MI_ERR_BAD_ARGUMENT;
+    const LaunchFn launch = d.bk == 64 ? row->deep[dtype] : row->twin[dtype];
+    return launch(c, plan.k_splits, needs_edge(c, d), stream);
 }
 
 // Re-packs an operand into K-contiguous rows of pitch kp (a multiple of 8), zero-padding columns K..kp-1.
@@ -938,8 +873,10 @@ struct BatchRequest {
     uint64_t a_stride, b_stride, c_stride;
 };
 
+// `attributes_only`: go through the plan this call would run and set the attributes of every GEMM kernel it would
+// launch, launching nothing (mi_matmul_mfma_prepare).  The helper kernels (fill, re-pack, sums) need no attribute.
 static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* workspace, size_t workspace_bytes, void* hip_stream,
-                    const TimelineRequest* timeline = nullptr, const BatchRequest* batch = nullptr)
+                    const TimelineRequest* timeline = nullptr, const BatchRequest* batch = nullptr, bool attributes_only = false)
 {
     if (const int st = check_modes(t, k_mode, tile)) {
         return st;
@@ -976,15 +913,16 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         return MI_ERR_UNSUPPORTED;
     }
     hipStream_t stream = as_stream(hip_stream);
+    p.c.attributes_only = attributes_only;
     if (p.repack_a) {
         p.c.a = (char*)workspace + p.ws_a;
-        if (const int st = repack(p.a_src, t->K, const_cast<void*>(p.c.a), stream)) {
+        if (const int st = attributes_only ? MI_OK : repack(p.a_src, t->K, const_cast<void*>(p.c.a), stream)) {
             return st;
         }
     }
     if (p.repack_b) {
         p.c.b = (char*)workspace + p.ws_b;
-        if (const int st = repack(p.b_src, t->K, const_cast<void*>(p.c.b), stream)) {
+        if (const int st = attributes_only ? MI_OK : repack(p.b_src, t->K, const_cast<void*>(p.c.b), stream)) {
             return st;
         }
     }
@@ -998,9 +936,8 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
     if (tile == MI_TILE_AUTO && plan.k_mode == MI_K_OUTPUT_STATIONARY && batch == nullptr && timeline == nullptr) {
         const Peel peel = plan_peeled(c, device_compute_units(), plan.cost_us);
         if (peel.on) {
-            const bool f16 = t->ab_dtype == MI_F16;
             auto launch = [&](const Canonical& part, const Plan& part_plan) -> int {
-                if (part_plan.k_splits > 1) {
+                if (part_plan.k_splits > 1 && !attributes_only) {
                     // a strip whose K partitions meet through atomics: its part of C starts at zero
                     size_t blocks = ((size_t)part.M * part.N + 255) / 256;
                     blocks = blocks > 4096 ? 4096 : blocks;
@@ -1008,7 +945,7 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
                                        part.ldc);
                     MI_CHECK_LAUNCH();
                 }
-                return f16 ? launch_tile<MI_F16>(part, part_plan, stream) : launch_tile<MI_BF16>(part, part_plan, stream);
+                return launch_tile(t->ab_dtype, part, part_plan, stream);
             };
             if (const int st = launch(peel_interior(c, peel), peel.interior_plan)) {
                 return st;
@@ -1025,8 +962,8 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         Canonical k = c;
         k.c = (float*)((char*)workspace + partial_off);
         k.stream_k_workgroups = plan.workgroups;
-        const int st = t->ab_dtype == MI_F16 ? launch_tile<MI_F16>(k, plan, stream) : launch_tile<MI_BF16>(k, plan, stream);
-        return st ? st : stream_k_sum(k.c, c, plan, stream);
+        const int st = launch_tile(t->ab_dtype, k, plan, stream);
+        return st || attributes_only ? st : stream_k_sum(k.c, c, plan, stream);
     }
     if (plan.k_mode == MI_K_SPLIT_REDUCE) {
         // partition s of problem l stores its copy of C at partials[l][s]; the sum then writes the caller's C
@@ -1034,10 +971,10 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         k.c = (float*)((char*)workspace + partial_off);
         k.c_split_bytes = (uint64_t)c.M * c.N * 4;
         k.c_batch_bytes = k.c_split_bytes * plan.k_splits;
-        const int st = t->ab_dtype == MI_F16 ? launch_tile<MI_F16>(k, plan, stream) : launch_tile<MI_BF16>(k, plan, stream);
-        return st ? st : reduce_partials(k.c, c, plan.k_splits, stream);
+        const int st = launch_tile(t->ab_dtype, k, plan, stream);
+        return st || attributes_only ? st : reduce_partials(k.c, c, plan.k_splits, stream);
     }
-    if (plan.k_splits > 1) {
+    if (plan.k_splits > 1 && !attributes_only) {
         // partial sums are atomically added: C must start at zero (gemm/gemm_sm90.cu:1208-1210).  A fill kernel,
         // not hipMemsetAsync, so the call stays safe to capture into a HIP graph.
         const size_t per_problem = (size_t)c.M * c.N;
@@ -1051,10 +988,7 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
             MI_CHECK_LAUNCH();
         }
     }
-    if (t->ab_dtype == MI_F16) {
-        return launch_tile<MI_F16>(c, plan, stream);
-    }
-    return launch_tile<MI_BF16>(c, plan, stream);
+    return launch_tile(t->ab_dtype, c, plan, stream);
 }
 
 }  // namespace mi_gemm
@@ -1342,7 +1276,7 @@ int mi_matmul_mfma_workspace_bytes_for(const mi_gemm_tensors* t, int k_mode, int
             // the forced mode runs with whatever holds the parts of the smallest tile that can be streamed
             size_t least = SIZE_MAX;
             const int cus = device_compute_units();
-            for (int tl = tile == MI_TILE_AUTO ? MI_TILE_256x256 : tile; tl <= (tile == MI_TILE_AUTO ? MI_TILE_COUNT_ - 1 : tile); ++tl) {
+            for (int tl = tile == MI_TILE_AUTO ? 1 : tile; tl <= (tile == MI_TILE_AUTO ? MI_TILE_COUNT_ - 1 : tile); ++tl) {
                 const uint32_t wgs = stream_k_workgroups(p.c, tl, cus);
                 if (wgs > 0 && stream_k_bytes(tl, p.c.K, wgs) < least) {
                     least = stream_k_bytes(tl, p.c.K, wgs);
@@ -1353,7 +1287,7 @@ int mi_matmul_mfma_workspace_bytes_for(const mi_gemm_tensors* t, int k_mode, int
     }
     if (k_mode == MI_K_SPLIT_REDUCE && plan.k_splits > 1) {
         // the forced mode runs with any room that holds the fewest copies some tile can be split into
-        const int tile_lo = tile == MI_TILE_AUTO ? MI_TILE_256x256 : tile;
+        const int tile_lo = tile == MI_TILE_AUTO ? 1 : tile;
         const int tile_hi = tile == MI_TILE_AUTO ? MI_TILE_COUNT_ - 1 : tile;
         for (uint32_t splits = 2; splits <= plan.k_splits; ++splits) {
             bool fits = false;
@@ -1382,6 +1316,20 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
     return run_mfma(t, k_mode, tile, d_workspace, d_workspace ? workspace_bytes : 0, hip_stream);
 }
 
+int mi_matmul_mfma_prepare(const mi_gemm_tensors* t, int k_mode, int tile, size_t workspace_bytes)
+{
+    if (const int st = check_modes(t, k_mode, tile)) {
+        return st;
+    }
+    // the plan depends on the workspace's size only (and on its presence): a stand-in address with the alignment the
+    // call asks for keeps the planner on the path the real call takes; nothing is read or written through it
+    void* const stand_in = workspace_bytes ? reinterpret_cast<void*>(uintptr_t(256)) : nullptr;
+    if (workspace_bytes && prepare(*t).ws_bytes > workspace_bytes) {
+        return MI_ERR_WORKSPACE;
+    }
+    return run_mfma(t, k_mode, tile, stand_in, workspace_bytes, nullptr, nullptr, nullptr, true);
+}
+
 int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream)
 {
     if (const int st = check_modes(t, k_mode, tile)) {
@@ -1398,25 +1346,39 @@ int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* 
     return run_mfma(t, k_mode, tile, ptr, STATIC_SCRATCH_BYTES, hip_stream);
 }
 
+int mi_tile_count(void)
+{
+    return MI_TILE_COUNT_;
+}
+
 const char* mi_tile_name(int tile)
 {
-    switch (tile) {
-    case MI_TILE_AUTO: return "auto";
-    case MI_TILE_256x256: return "256x256";
-    case MI_TILE_256x128: return "256x128";
-    case MI_TILE_128x128: return "128x128";
-    case MI_TILE_64x128: return "64x128";
-    case MI_TILE_192x256: return "192x256";
-    case MI_TILE_224x256: return "224x256";
-    case MI_TILE_160x256: return "160x256";
-    case MI_TILE_224x128: return "224x128";
-    case MI_TILE_160x128: return "160x128";
-    case MI_TILE_256x192: return "256x192";
-    case MI_TILE_192x192: return "192x192";
-    case MI_TILE_192x128: return "192x128";
-    case MI_TILE_96x128: return "96x128";
+    if (tile == MI_TILE_AUTO) {
+        return "auto";
     }
-    return "unknown";
+    const TileRow* const row = tile_row(tile);
+    return row != nullptr ? row->name : "unknown";
+}
+
+int mi_tile_shape(int tile, uint32_t* out_bm, uint32_t* out_bn, int* out_workgroups_per_cu, int* out_has_32_deep_twin)
+{
+    const TileRow* const row = tile_row(tile);
+    if (row == nullptr) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    if (out_bm) {
+        *out_bm = row->bm;
+    }
+    if (out_bn) {
+        *out_bn = row->bn;
+    }
+    if (out_workgroups_per_cu) {
+        *out_workgroups_per_cu = row->per_cu;
+    }
+    if (out_has_32_deep_twin) {
+        *out_has_32_deep_twin = row->twin[0] != nullptr ? 1 : 0;
+    }
+    return MI_OK;
 }
 
 const char* mi_k_mode_name(int k_mode)

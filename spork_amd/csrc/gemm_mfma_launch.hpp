@@ -75,12 +75,14 @@ struct Canonical {
     uint32_t timeline_slots = 0;
     uint32_t timeline_workgroups = 0;   // capacity of the stamp buffer in workgroups
     uint32_t* launched_workgroups = nullptr;  // out: grid size of the launch
+    // set the kernel's attributes (the dynamic LDS opt-in) and launch nothing: see mi_matmul_mfma_prepare
+    bool attributes_only = false;
 };
 
 constexpr uint32_t GROUP_M = 4;  // tile-rows per raster group (see map_work)
 
 template <int DTYPE, typename Cfg, bool ATOMIC, bool EDGE, bool STREAM = false, int ONCE = 0>
-int launch_kernel(const GemmArgs& args, uint32_t grid, hipStream_t stream)
+int launch_kernel(const GemmArgs& args, uint32_t grid, hipStream_t stream, bool attributes_only)
 {
     // dynamic LDS above the 64 KB default needs an opt-in once per device (gemm/gemm_sm80.cu:473-475)
     static std::atomic<bool> attr_set[64];  // per kernel instantiation; setting the attribute twice is harmless
@@ -92,6 +94,9 @@ int launch_kernel(const GemmArgs& args, uint32_t grid, hipStream_t stream)
         if (dev >= 0 && dev < 64) {
             attr_set[dev].store(true, std::memory_order_release);
         }
+    }
+    if (attributes_only) {
+        return MI_OK;
     }
     hipLaunchKernelGGL((gemm_tn_kernel<DTYPE, Cfg, ATOMIC, EDGE, STREAM, ONCE>), dim3(grid), dim3(Cfg::NTHREADS),
                        Cfg::LDS_BYTES, stream, args);
@@ -158,32 +163,32 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
     // workgroup at a time and the hardware dispatcher hands it the next one as soon as the previous one has ended.
     if constexpr (Cfg::BK == 64) {
         if (stream_k) {
-            return launch_kernel<DTYPE, Cfg, false, false, true>(args, grid, stream);
+            return launch_kernel<DTYPE, Cfg, false, false, true>(args, grid, stream, c.attributes_only);
         }
     }
     if (k_splits > 1 && c.c_split_bytes == 0) {
         if constexpr (Cfg::BK == 64) {
             if (!edge && c.read_once == 1 && c.batches == 1) {
-                return launch_kernel<DTYPE, Cfg, true, false, false, 1>(args, grid, stream);
+                return launch_kernel<DTYPE, Cfg, true, false, false, 1>(args, grid, stream, c.attributes_only);
             }
             if (!edge && c.read_once == 2 && c.batches == 1) {
-                return launch_kernel<DTYPE, Cfg, true, false, false, 2>(args, grid, stream);
+                return launch_kernel<DTYPE, Cfg, true, false, false, 2>(args, grid, stream, c.attributes_only);
             }
         }
-        return edge ? launch_kernel<DTYPE, Cfg, true, true>(args, grid, stream)
-                    : launch_kernel<DTYPE, Cfg, true, false>(args, grid, stream);
+        return edge ? launch_kernel<DTYPE, Cfg, true, true>(args, grid, stream, c.attributes_only)
+                    : launch_kernel<DTYPE, Cfg, true, false>(args, grid, stream, c.attributes_only);
     }
     if constexpr (Cfg::BK == 64) {
         // (which launches qualify is the host planner's decision: read_once_operand)
         if (!edge && c.read_once == 1 && c.batches == 1) {
-            return launch_kernel<DTYPE, Cfg, false, false, false, 1>(args, grid, stream);
+            return launch_kernel<DTYPE, Cfg, false, false, false, 1>(args, grid, stream, c.attributes_only);
         }
         if (!edge && c.read_once == 2 && c.batches == 1) {
-            return launch_kernel<DTYPE, Cfg, false, false, false, 2>(args, grid, stream);
+            return launch_kernel<DTYPE, Cfg, false, false, false, 2>(args, grid, stream, c.attributes_only);
         }
     }
-    return edge ? launch_kernel<DTYPE, Cfg, false, true>(args, grid, stream)
-                : launch_kernel<DTYPE, Cfg, false, false>(args, grid, stream);
+    return edge ? launch_kernel<DTYPE, Cfg, false, true>(args, grid, stream, c.attributes_only)
+                : launch_kernel<DTYPE, Cfg, false, false>(args, grid, stream, c.attributes_only);
 }
 
 #define MI_GEMM_DECLARE_CFG(Cfg)                                                                    \
@@ -192,5 +197,66 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
 #define MI_GEMM_INSTANTIATE_CFG(Cfg)                                                         \
     template int launch_cfg<MI_F16, Cfg>(const Canonical&, uint32_t, bool, hipStream_t);    \
     template int launch_cfg<MI_BF16, Cfg>(const Canonical&, uint32_t, bool, hipStream_t);
+
+// ---- the one table of the tile family.  Everything that depends on which tiles exist is generated from it: tile
+// dimensions, names, the dispatch to a configuration's launcher, the planner's cost constants, the exported
+// mi_tile_count / mi_tile_name / mi_tile_shape that bindings, tests and the host driver enumerate.  Adding a tile is a
+// `using Cfg... = TileCfg<...>` line above, a row here (plus a line in MI_TILE_TWINS if it has a 32-deep twin), an
+// enumerator in mi_gemm.h and a gemm_mfma_inst_*.hip that instantiates it.
+//
+// Columns: ABI code, name, 64-deep configuration, 32-deep twin (or NoTwin: a K that is only a multiple of 32 then runs
+// the range-checked build with a half-empty last slot), then the planner's measured constants on MI355X
+// at the clock the chip sustains under MFMA load:
+//   us_k64      main-loop time per 64-deep K step with every CU busy (of a pair of workgroups for a tile whose ring
+//               lets two share a CU)
+//   fixed_us    per-workgroup cost outside the main loop (dispatch, ring fill, epilogue), a whole round ending together
+//   short_us    the same for K <= 384 and at least two rounds of the largest tile, where a launch is a stream of C stores
+//               (measured on 8192^2 x 64..384, 16384^2 x 128, 32768 x 65536 x 48)
+//   per_cu      workgroups that share a CU
+//   alone_k64 / alone_us   us_k64 / fixed_us of a workgroup that has its CU to itself (differs for per_cu = 2 only)
+//   max_k       the planner leaves the tile to callers that force it above this K (0: no limit).  192x128, two per CU,
+//               wins where workgroups are short-lived: ahead by 13 % at K = 512 and 1024, level at 1408, behind by 8
+//               to 10 % at 1536 and 2048 (3000 x 11008 x 4096: 253 us against 214 us)
+#define MI_TILE_TABLE(ROW)                                                                                          \
+    ROW(MI_TILE_256x256, "256x256", Cfg256x256, Cfg256x256k32, 1.33, 15.0, 17.4, 1, 1.33, 15.0, 0)             \
+    ROW(MI_TILE_256x128, "256x128", Cfg256x128, Cfg256x128k32, 0.73, 10.0, 7.2, 1, 0.73, 10.0, 0)              \
+    ROW(MI_TILE_128x128, "128x128", Cfg128x128, Cfg128x128k32, 0.44, 7.0, 3.0, 1, 0.44, 7.0, 0)                \
+    ROW(MI_TILE_64x128, "64x128", Cfg64x128, Cfg64x128k32, 0.25, 6.0, 2.8, 1, 0.25, 6.0, 0)                    \
+    ROW(MI_TILE_192x256, "192x256", Cfg192x256, Cfg192x256k32, 1.03, 13.0, 8.5, 1, 1.03, 13.0, 0)              \
+    ROW(MI_TILE_224x256, "224x256", Cfg224x256, NoTwin, 1.16, 13.5, 13.0, 1, 1.16, 13.5, 0)                         \
+    ROW(MI_TILE_160x256, "160x256", Cfg160x256, NoTwin, 0.86, 12.0, 7.5, 1, 0.86, 12.0, 0)                          \
+    ROW(MI_TILE_224x128, "224x128", Cfg224x128, NoTwin, 0.64, 9.5, 6.5, 1, 0.64, 9.5, 0)                            \
+    ROW(MI_TILE_160x128, "160x128", Cfg160x128, NoTwin, 0.48, 8.5, 4.0, 1, 0.48, 8.5, 0)                            \
+    ROW(MI_TILE_256x192, "256x192", Cfg256x192, NoTwin, 1.02, 13.0, 10.0, 1, 1.02, 13.0, 0)                         \
+    ROW(MI_TILE_192x192, "192x192", Cfg192x192, NoTwin, 0.755, 18.5, 8.0, 1, 0.755, 18.5, 0)                        \
+    /* two per CU: the times of such a pair, measured on 7072 x 7352 x 1024, 6144 x 4096 x 1024, 8192^2 x 2048 and    \
+       8192^2 x 256 (126, 53, 246, 65 us) */                                                                        \
+    ROW(MI_TILE_192x128, "192x128", Cfg192x128, NoTwin, 1.0, 9.0, 8.0, 2, 0.85, 12.0, 1536)                         \
+    ROW(MI_TILE_96x128, "96x128", Cfg96x128, NoTwin, 0.36, 6.5, 2.9, 1, 0.36, 6.5, 0)
+#define MI_TILE_TWINS(X) X(Cfg256x256k32) X(Cfg256x128k32) X(Cfg128x128k32) X(Cfg64x128k32) X(Cfg192x256k32)
+
+using LaunchFn = int (*)(const Canonical&, uint32_t, bool, hipStream_t);
+
+struct NoTwin {};
+template <typename Cfg>
+struct Launchers {
+    static constexpr LaunchFn f16 = &launch_cfg<MI_F16, Cfg>, bf16 = &launch_cfg<MI_BF16, Cfg>;
+};
+template <>
+struct Launchers<NoTwin> {
+    static constexpr LaunchFn f16 = nullptr, bf16 = nullptr;
+};
+
+struct TileRow {
+    int code;
+    const char* name;
+    uint32_t bm, bn;
+    LaunchFn deep[2];  // 64-deep configuration, by element type (MI_F16, MI_BF16)
+    LaunchFn twin[2];  // 32-deep twin, or null
+    double us_k64, fixed_us, short_us;
+    int per_cu;
+    double alone_k64, alone_us;
+    uint32_t max_k;
+};
 
 }  // namespace mi_gemm

@@ -26,6 +26,29 @@ static void* device_alloc(size_t bytes)
     return p;
 }
 
+// What the harness shows of a wrong element: [baseline, tested] pairs of the 5 x 5 elements around it, the wrong one in
+// bold (gemm/gemm_test.cu:98-120, which prints from the device; here the rows are copied back and printed by the host).
+static void print_tensor_neighborhood(const float* d_a, const float* d_b, uint32_t rows, uint32_t cols, uint32_t y, uint32_t x)
+{
+    if (y >= rows || x >= cols) {
+        return;
+    }
+    const uint32_t y_min = y < 2 ? 0u : y - 2, y_max = y + 2 >= rows ? rows - 1u : y + 2;
+    const uint32_t x_min = x < 2 ? 0u : x - 2, x_max = x + 2 >= cols ? cols - 1u : x + 2;
+    const uint32_t width = x_max - x_min + 1;
+    float a[5], b[5];
+    for (uint32_t cy = y_min; cy <= y_max; ++cy) {
+        const size_t first = size_t(cy) * cols + x_min;
+        gpu_check(mi_rt_memcpy_d2h(a, d_a + first, sizeof(float) * width), "read baseline row");
+        gpu_check(mi_rt_memcpy_d2h(b, d_b + first, sizeof(float) * width), "read tested row");
+        for (uint32_t cx = x_min; cx <= x_max; ++cx) {
+            const bool it = cy == y && cx == x;
+            printf("%s[%6g, %5g]%s  ", it ? "\x1b[1m" : "", a[cx - x_min], b[cx - x_min], it ? "\x1b[0m" : "");
+        }
+        printf("\n");
+    }
+}
+
 int gemm_test(TestParams params, gpu_stream_t stream)
 {
     StreamWorkspace stream_ws{stream};
@@ -90,45 +113,6 @@ int gemm_test(TestParams params, gpu_stream_t stream)
               case AlgorithmCode::mi355_auto:
                 matmul_mi355(t, MI_K_AUTO, MI_TILE_AUTO, stream);
                 break;
-              case AlgorithmCode::mi355_256x256:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_256x256, stream);
-                break;
-              case AlgorithmCode::mi355_256x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_256x128, stream);
-                break;
-              case AlgorithmCode::mi355_128x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_128x128, stream);
-                break;
-              case AlgorithmCode::mi355_64x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_64x128, stream);
-                break;
-              case AlgorithmCode::mi355_192x256:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_192x256, stream);
-                break;
-              case AlgorithmCode::mi355_224x256:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_224x256, stream);
-                break;
-              case AlgorithmCode::mi355_160x256:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_160x256, stream);
-                break;
-              case AlgorithmCode::mi355_224x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_224x128, stream);
-                break;
-              case AlgorithmCode::mi355_160x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_160x128, stream);
-                break;
-              case AlgorithmCode::mi355_256x192:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_256x192, stream);
-                break;
-              case AlgorithmCode::mi355_192x192:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_192x192, stream);
-                break;
-              case AlgorithmCode::mi355_192x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_192x128, stream);
-                break;
-              case AlgorithmCode::mi355_96x128:
-                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, MI_TILE_96x128, stream);
-                break;
               case AlgorithmCode::mi355_split_k:
                 matmul_mi355(t, MI_K_SPLIT, MI_TILE_AUTO, stream);
                 break;
@@ -149,6 +133,9 @@ int gemm_test(TestParams params, gpu_stream_t stream)
                 matmul_mi355_any_layout(t_row, stream_ws);
                 break;
               }
+              default:  // one of the library's tiles, forced
+                matmul_mi355(t, MI_K_OUTPUT_STATIONARY, forced_tile_of(algo), stream);
+                break;
             }
             if (launch_i >= warmup_count) {
                 test_events[test_i + 1] = new_event();
@@ -168,16 +155,19 @@ int gemm_test(TestParams params, gpu_stream_t stream)
         memcpy(&max_diff, &result[1], 8);
         memcpy(&max_ref, &result[2], 8);
         const double rel_err = max_ref > 0 ? max_diff / max_ref : max_diff;
+        const bool nonneg_data = params.test_data_code_A <= TestDataCode::tiled_numbers && params.test_data_code_B <= TestDataCode::tiled_numbers;
+        const bool failed = !(rel_err <= 1e-3) || (nonneg_data && result[0] != UINT64_MAX);
         if (result[0] != UINT64_MAX) {
             // the reference's ratio rule (gemm/gemm_test.cu:138-147); informative for signed data, where elements
             // near zero fail it through cancellation alone
+            const uint32_t y = static_cast<uint32_t>(result[0] >> 32), x = static_cast<uint32_t>(result[0]);
             printf("TestParams{%u,%u,%u, %i,%i} \x1b[1m[%u,%u]\x1b[0m first of %llu elements outside ratio 1+1/32\n", params.M,
-                   params.N, params.K, static_cast<int>(params.test_data_code_A), static_cast<int>(params.test_data_code_B),
-                   static_cast<uint32_t>(result[0] >> 32), static_cast<uint32_t>(result[0]),
+                   params.N, params.K, static_cast<int>(params.test_data_code_A), static_cast<int>(params.test_data_code_B), y, x,
                    static_cast<unsigned long long>(result[3]));
+            if (failed) {
+                print_tensor_neighborhood(d_c_baseline, d_c_tested, params.M, params.N, y, x);
+            }
         }
-        const bool nonneg_data = params.test_data_code_A <= TestDataCode::tiled_numbers && params.test_data_code_B <= TestDataCode::tiled_numbers;
-        const bool failed = !(rel_err <= 1e-3) || (nonneg_data && result[0] != UINT64_MAX);
         failures += failed;
 
         for (uint32_t test_i = 0; test_i < test_count; ++test_i) {
@@ -203,7 +193,7 @@ int gemm_test(TestParams params, gpu_stream_t stream)
         fflush(stdout);
     };
 
-    for (uint32_t bit_index = 0; bit_index < algorithm_count; ++bit_index) {
+    for (uint32_t bit_index = 0; bit_index < algorithm_count() && bit_index < algorithm_max_count; ++bit_index) {
         if ((params.algorithm_code_bits >> bit_index & 1) == 0) {
             continue;
         }

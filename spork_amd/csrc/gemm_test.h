@@ -2,6 +2,7 @@
 #pragma once
 
 #include <stdint.h>
+#include <stdio.h>
 
 #include "gpu_tensor.h"
 
@@ -15,39 +16,49 @@ enum class TestDataCode
     normal = MI_DATA_NORMAL,    // normal(0,1) * data_param
 };
 
-// gemm/gemm_test.h:13-38: one bit per algorithm raced against the baseline.
+// gemm/gemm_test.h:13-38: one bit per algorithm raced against the baseline.  The fixed algorithms come first; after
+// them one "this tile, output stationary" algorithm per tile of the library's family (index algorithm_fixed_count +
+// tile code - 1): the list is whatever mi_tile_count() / mi_tile_name() report, so a new tile shows up here by itself.
 enum class AlgorithmCode
 {
     mfma_direct,          // one MFMA tile per wave straight from global memory
     mi355_auto,           // planner picks tile and K mode
-    mi355_256x256,        // output stationary, fixed tile
-    mi355_256x128,
-    mi355_128x128,
-    mi355_64x128,
-    mi355_192x256,
-    mi355_224x256,
-    mi355_160x256,
-    mi355_224x128,
-    mi355_160x128,
-    mi355_256x192,
-    mi355_192x192,
-    mi355_192x128,
-    mi355_96x128,
     mi355_split_k,        // planner picks the tile, K split forced
     mi355_row_major_b,    // B given K x N row-major (the baseline's own call): re-packed through the workspace
     mi355_auto_ws,        // planner with a workspace at hand: K partitions may be summed from copies of C
     mi355_split_k_sum,    // K split forced, partitions summed from copies of C in the workspace (no atomics)
     mi355_stream_k,       // stream-K forced: equal runs of (tile, K tile) pairs, parts summed from the workspace
     hipblaslt,            // vendor comparator (the cuBLAS / CUTLASS rows of gemm/gemm_test.h:19-20)
+    first_forced_tile,    // + (tile code - 1)
 };
 
-constexpr uint32_t algorithm_count = 1u + static_cast<uint32_t>(AlgorithmCode::hipblaslt);
+constexpr uint32_t algorithm_fixed_count = static_cast<uint32_t>(AlgorithmCode::first_forced_tile);
+constexpr uint32_t algorithm_max_count = 64;  // bits of the selection mask
 
-inline uint32_t algorithm_code_bit(AlgorithmCode code)
+inline uint32_t algorithm_count()
 {
-    return 1u << static_cast<uint32_t>(code);
+    return algorithm_fixed_count + static_cast<uint32_t>(mi_tile_count() - 1);
 }
 
+inline uint64_t algorithm_code_bit(AlgorithmCode code)
+{
+    return uint64_t(1) << static_cast<uint32_t>(code);
+}
+
+// the algorithm that forces tile `tile` (an MI_TILE_* code other than MI_TILE_AUTO), output stationary
+inline AlgorithmCode forced_tile_algorithm(int tile)
+{
+    return static_cast<AlgorithmCode>(algorithm_fixed_count + static_cast<uint32_t>(tile - 1));
+}
+
+// 0 for the fixed algorithms, else the tile code the algorithm forces
+inline int forced_tile_of(AlgorithmCode code)
+{
+    const uint32_t index = static_cast<uint32_t>(code);
+    return index < algorithm_fixed_count ? 0 : static_cast<int>(index - algorithm_fixed_count) + 1;
+}
+
+// (the returned pointer is valid until the next call from the same thread)
 inline const char* algorithm_name(AlgorithmCode code)
 {
     switch (code) {
@@ -55,32 +66,6 @@ inline const char* algorithm_name(AlgorithmCode code)
         return "mfma_direct";
       case AlgorithmCode::mi355_auto:
         return "mi355 (auto)";
-      case AlgorithmCode::mi355_256x256:
-        return "mi355 256x256 (output stationary)";
-      case AlgorithmCode::mi355_256x128:
-        return "mi355 256x128 (output stationary)";
-      case AlgorithmCode::mi355_128x128:
-        return "mi355 128x128 (output stationary)";
-      case AlgorithmCode::mi355_64x128:
-        return "mi355 64x128 (output stationary)";
-      case AlgorithmCode::mi355_192x256:
-        return "mi355 192x256 (output stationary)";
-      case AlgorithmCode::mi355_224x256:
-        return "mi355 224x256 (output stationary)";
-      case AlgorithmCode::mi355_160x256:
-        return "mi355 160x256 (output stationary)";
-      case AlgorithmCode::mi355_224x128:
-        return "mi355 224x128 (output stationary)";
-      case AlgorithmCode::mi355_160x128:
-        return "mi355 160x128 (output stationary)";
-      case AlgorithmCode::mi355_256x192:
-        return "mi355 256x192 (output stationary)";
-      case AlgorithmCode::mi355_192x192:
-        return "mi355 192x192 (output stationary)";
-      case AlgorithmCode::mi355_192x128:
-        return "mi355 192x128, two per CU (output stationary)";
-      case AlgorithmCode::mi355_96x128:
-        return "mi355 96x128 (output stationary)";
       case AlgorithmCode::mi355_split_k:
         return "mi355 (split k)";
       case AlgorithmCode::mi355_row_major_b:
@@ -93,8 +78,17 @@ inline const char* algorithm_name(AlgorithmCode code)
         return "mi355 (stream k)";
       case AlgorithmCode::hipblaslt:
         return "hipBLASLt";
+      default:
+        break;
     }
-    return "unknown";
+    const int tile = forced_tile_of(code);
+    int per_cu = 1;
+    if (tile < 1 || mi_tile_shape(tile, nullptr, nullptr, &per_cu, nullptr) != MI_OK) {
+        return "unknown";
+    }
+    static thread_local char text[64];
+    snprintf(text, sizeof text, "mi355 %s%s (output stationary)", mi_tile_name(tile), per_cu == 2 ? ", two per CU" : "");
+    return text;
 }
 
 // gemm/gemm_test.h:100-105, with the element type and the distribution parameter added.
@@ -102,10 +96,10 @@ struct TestParams
 {
     uint32_t M, N, K;
     TestDataCode test_data_code_A, test_data_code_B;
-    uint32_t algorithm_code_bits;
+    uint64_t algorithm_code_bits;
     int ab_dtype;        // MI_F16 | MI_BF16
     double data_param;   // for TestDataCode::uniform / normal
-    double* out_ms = nullptr;  // optional, algorithm_count entries: the reported time of each algorithm that ran
+    double* out_ms = nullptr;  // optional, algorithm_count() entries: the reported time of each algorithm that ran
 };
 
 // Runs every selected algorithm 25 times, compares each against the baseline kernel on the device and prints one line

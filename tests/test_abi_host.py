@@ -107,12 +107,43 @@ def test_supports_predicate():
     assert not S.matmul_mfma_supports(_t(256, 256, 256, a_col_major=1))
     assert not S.matmul_mfma_supports(_t(256, 256, 256, b_col_major=0))
     assert not S.matmul_mfma_supports(_t(256, 256, 256, a=260))       # A not 16-byte aligned
+    # the range-checked build counts rows in signed 32-bit integers: 2^31 rows and more are refused, on either side
+    assert S.matmul_mfma_supports(_t((1 << 31) - 8, 8, 8))
+    assert not S.matmul_mfma_supports(_t(1 << 31, 8, 8))
+    assert not S.matmul_mfma_supports(_t(8, 1 << 31, 8, c_col_major=1))
+    assert not S.matmul_mfma_supports(_t(8, 1 << 21, 8))              # N beyond a descriptor's 32-bit offsets
     # explicit tiles
     assert S.matmul_mfma_supports(_t(256, 256, 64), S.K_OUTPUT_STATIONARY, S.TILE_256x256)
     assert S.matmul_mfma_supports(_t(128, 256, 64), S.K_OUTPUT_STATIONARY, S.TILE_256x256)
     # a single K tile cannot be split: MI_K_SPLIT then degenerates to one partition (no atomics)
     assert S.matmul_mfma_plan(_t(256, 256, 64), S.K_SPLIT, S.TILE_256x256)["k_splits"] == 1
     assert S.matmul_mfma_plan(_t(256, 256, 128), S.K_SPLIT, S.TILE_256x256)["k_splits"] == 2
+
+
+def test_tile_family_is_enumerated_from_the_library():
+    """One table in the library defines the tile family; the binding's TILE_* names come from the header's enumerators
+    and shapes, names and the count from mi_tile_count / mi_tile_name / mi_tile_shape: they must agree."""
+    tiles = S.tiles()
+    assert len(tiles) == S.tile_count() - 1 == len(S.TILE_CODES) - 1
+    for t in tiles:
+        assert S.TILE_CODES[f"TILE_{t['name']}"] == t["code"]
+        assert t["name"] == f"{t['bm']}x{t['bn']}" and t["workgroups_per_cu"] in (1, 2)
+        # every tile is accepted when forced on a problem of whole tiles, and named by the plan
+        plan = S.matmul_mfma_plan(_t(2 * t["bm"], 3 * t["bn"], 256), S.K_OUTPUT_STATIONARY, t["code"])
+        assert plan["tile"] == t["name"] and plan["tile_code"] == t["code"]
+    assert S.lib().mi_tile_name(0) == b"auto" and S.lib().mi_tile_name(S.tile_count()) == b"unknown"
+    assert S.lib().mi_tile_shape(0, None, None, None, None) == 2
+    assert S.lib().mi_tile_shape(S.tile_count(), None, None, None, None) == 2
+    assert [t["name"] for t in tiles if t["has_32_deep_twin"]] == ["256x256", "256x128", "128x128", "64x128", "192x256"]
+    assert [t["name"] for t in tiles if t["workgroups_per_cu"] == 2] == ["192x128"]
+
+
+def test_prepare_entry_validates_like_the_call_it_prepares():
+    lib = S.lib()
+    assert lib.mi_matmul_mfma_prepare(None, S.K_AUTO, S.TILE_AUTO, 0) == 2
+    assert lib.mi_matmul_mfma_prepare(C.byref(_t(256, 256, 256)), 9, S.TILE_AUTO, 0) == 2
+    assert lib.mi_matmul_mfma_prepare(C.byref(_t(256, 256, 100)), S.K_AUTO, S.TILE_AUTO, 0) == 1       # needs re-packing
+    assert lib.mi_matmul_mfma_prepare(C.byref(_t(256, 256, 100)), S.K_AUTO, S.TILE_AUTO, 4096) == 3    # too little room
 
 
 def test_workspace_size_query():

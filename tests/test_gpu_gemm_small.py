@@ -4,6 +4,7 @@ import pytest
 import torch
 
 import helpers as H
+import spork_amd as S
 
 pytestmark = pytest.mark.gpu
 
@@ -69,8 +70,8 @@ def test_baseline_all_layouts_ragged(gpu, oracle, dtype, layout):
     assert H.rel_err(got, ref) < 1e-5
 
 
-TILES = [(1, 256, 256), (2, 256, 128), (3, 128, 128), (4, 64, 128), (5, 192, 256), (6, 224, 256), (7, 160, 256),
-         (8, 224, 128), (9, 160, 128), (10, 256, 192), (11, 192, 192), (12, 192, 128), (13, 96, 128)]
+# every tile of the family, as the library itself lists it: (code, rows, columns)
+TILES = [pytest.param(t["code"], t["bm"], t["bn"], id=t["name"]) for t in S.tiles()]
 
 
 @pytest.mark.parametrize("dtype", [0, 1])

@@ -67,3 +67,69 @@ def test_entry_points_replay_correctly_from_a_graph(gpu, name):
             assert H.rel_err(got, want.astype(np.float64)) < 1e-5, (name, replay)   # atomics: order of additions varies
         else:
             np.testing.assert_array_equal(got, want, err_msg=f"{name} replay {replay}")
+
+
+_PREPARED_CAPTURE = r"""
+import sys
+import numpy as np
+import torch
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests")
+import helpers as H
+import spork_amd as S
+
+torch.cuda.set_device(0)
+failures = 0
+# name: (M, N, K, k_mode, tile, workspace bytes; -1: the library's own scratch array)
+cases = {"output_stationary": (512, 768, 1024, S.K_OUTPUT_STATIONARY, S.TILE_256x256, 0),
+         "split_k_workspace_sum": (256, 384, 4096, S.K_SPLIT_REDUCE, S.TILE_128x128, 1 << 24),
+         "ragged_edge_build": (300, 504, 1000, S.K_AUTO, S.TILE_AUTO, 0),
+         "static_scratch": (256, 384, 4096, S.K_SPLIT_REDUCE, S.TILE_64x128, -1)}
+for name, (M, N, K, k_mode, tile, ws_bytes) in cases.items():
+    a, b = H.dev_u16(M, K), H.dev_u16(N, K)
+    c_graph, c_eager = H.poisoned_c(M, N), H.poisoned_c(M, N)
+    tg, te = H.tensors(M, N, K, a, b, c_graph, 1), H.tensors(M, N, K, a, b, c_eager, 1)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+
+    def call(t):
+        if ws_bytes < 0:
+            S.matmul_mfma_static(t, k_mode, tile, H.stream_handle())
+        elif ws_bytes:
+            S.matmul_mfma_ws(t, ws.data_ptr(), ws_bytes, k_mode, tile, H.stream_handle())
+        else:
+            S.matmul_mfma(t, k_mode, tile, H.stream_handle())
+
+    # no eager call first: only the prepare entry (and, for the static entry, the set-up call that looks up its array)
+    S.matmul_mfma_prepare(tg, k_mode, tile, S.STATIC_SCRATCH_BYTES if ws_bytes < 0 else ws_bytes)
+    if ws_bytes < 0:
+        S.lib().mi_rt_set_device(0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(tg)
+    for replay in range(3):
+        for t_, seed in ((a, 10 + replay), (b, 20 + replay)):
+            S.init_test_data(t_.data_ptr(), t_.shape[0], t_.shape[1], 4, t_ is b, 1, K ** -0.5, seed, H.stream_handle())
+        c_graph.view(torch.uint8).fill_(0x7D)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        call(te)
+        torch.cuda.synchronize()
+        same = np.array_equal(c_graph.cpu().numpy().view(np.uint32), c_eager.cpu().numpy().view(np.uint32))
+        print(f"{name} replay {replay}: {'same bits' if same else 'DIFFERENT'}", flush=True)
+        failures += not same
+sys.exit(1 if failures else 0)
+"""
+
+
+def test_capture_preceded_only_by_prepare(gpu):
+    """A first call made inside a capture works when mi_matmul_mfma_prepare has run: in a process of its own, so that no
+    earlier test has launched (and thereby set up) the kernels."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", _PREPARED_CAPTURE, root], capture_output=True, text=True, timeout=110)
+    print(out.stdout[-3000:], out.stderr[-3000:], flush=True)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
+    assert out.stdout.count("same bits") == 12
