@@ -7,6 +7,7 @@
 //   gemm --rounds   the same idea re-derived for this chip: tile counts around multiples of its CU count
 //   gemm --versus llm|random    the planner against hipBLASLt over many shapes, with a summary table
 //   gemm --one M N K [f16|bf16] [data style 1..5] [param]    the planner (without and with workspace) and hipBLASLt on one shape
+//   gemm --kmodes M N K [f16|bf16] [style] [param]  one size: the planner, each K mode forced, hipBLASLt
 //   gemm --timeline M N K [f16|bf16] [tile code]    in-kernel timeline of one launch
 //   gemm --ceiling  what a register-only MFMA loop sustains on the benchmark's operand values
 #include <math.h>
@@ -24,7 +25,8 @@ int main(int argc, char** argv)
     const bool sweep = argc > 1 && strcmp(argv[1], "--sweep") == 0;
     const bool rounds = argc > 1 && strcmp(argv[1], "--rounds") == 0;
     const bool versus = argc > 2 && strcmp(argv[1], "--versus") == 0;
-    const bool one = argc > 1 && strcmp(argv[1], "--one") == 0;
+    const bool kmodes = argc > 1 && strcmp(argv[1], "--kmodes") == 0;  // --one with every K mode as a row of its own
+    const bool one = kmodes || (argc > 1 && strcmp(argv[1], "--one") == 0);
     int device_count = 0;
     if (mi_rt_device_count(&device_count) != MI_OK || device_count == 0) {
         fprintf(stderr, "no GPU visible\n");
@@ -177,6 +179,10 @@ int main(int argc, char** argv)
         }
         keep_bits = algorithm_code_bit(AlgorithmCode::mi355_auto) | algorithm_code_bit(AlgorithmCode::mi355_auto_ws) |
                     algorithm_code_bit(AlgorithmCode::hipblaslt);
+        if (kmodes) {
+            keep_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum) |
+                         algorithm_code_bit(AlgorithmCode::mi355_stream_k);
+        }
         const int style = argc > 6 ? atoi(argv[6]) : 5;
         if (style < 1 || style > 5) {
             fprintf(stderr, "data style must be 1..5\n");

@@ -192,51 +192,93 @@ static size_t partial_bytes(const Canonical& c, uint32_t k_splits)
     return (size_t)c.M * c.N * 4 * k_splits * c.batches;
 }
 
-// Stream-K needs whole tiles, one problem, a C that takes 16-byte stores, and no more tiles than workgroups, so that a
-// workgroup's run of K tiles touches two tiles at most.  Returns the grid (0: not possible).
-static uint32_t stream_k_workgroups(const Canonical& c, int tile, int cus)
+// How a stream-K call (MI_K_STREAM) is laid out, the role of gemm/gemm_sm90.cu:1009-1030: the whole rounds of tiles
+// (`full_tiles`, a multiple of the workgroups one round holds) run the plain output-stationary kernel and store
+// straight into C; the `r` tiles that are left, fewer than a round, run as one stream-K launch of `g` workgroups (see
+// gemm_tn_kernel, STREAM) whose parts a last kernel sums into C.
+struct StreamKLayout {
+    uint32_t g;            // workgroups of the stream-K launch: one round
+    uint32_t full_tiles;   // tiles of the raster order's head that run output stationary
+    uint32_t r;            // tail tiles, 0 < r < g
+    uint32_t splits;       // S = g / r main partitions per tail tile
+    uint32_t lefts;        // L = g - r * S leftover workgroups
+    uint32_t k_tiles;      // KT
+    uint32_t main_k;       // Km: K tiles per tile covered by the main partitions (KT when there are no leftovers)
+    uint32_t bm, bn;
+    uint32_t slots() const { return r * splits + (lefts ? lefts + r - 1 : 0); }
+    size_t bytes() const { return (size_t)slots() * bm * bn * 4; }
+    uint32_t main_len() const { return (main_k + splits - 1) / splits; }                               // longest main partition
+    uint32_t left_len() const { return lefts ? (uint32_t)(((uint64_t)r * (k_tiles - main_k) + lefts - 1) / lefts) : 0; }
+    uint32_t left_parts() const  // most parts one leftover workgroup stores
+    {
+        const uint32_t kr = k_tiles - main_k;
+        return lefts ? (left_len() + kr - 2) / kr + 1 : 0;
+    }
+};
+
+// Stream-K needs whole tiles, one problem, a C that takes 16-byte stores, and a tile count that does not fill whole
+// rounds.  Returns false when the mode does not apply.
+static bool stream_k_layout(const Canonical& c, int tile, int cus, StreamKLayout& sk)
 {
     TileDims d;
-    if (!tile_dims(tile, c.K, d) || d.bk != 64 || c.M % d.bm || c.N % d.bn || c.K % 64 || c.batches != 1 ||
-        (uintptr_t)c.c % 16) {
-        return 0;
+    const TileRow* const row = tile_row(tile);
+    if (row == nullptr || !tile_dims(tile, c.K, d) || d.bk != 64 || c.M % d.bm || c.N % d.bn || c.K % 64 || c.batches != 1 ||
+        (uintptr_t)c.c % 16 || c.ldc % 4 || c.K == 0) {
+        return false;
     }
-    const uint64_t tiles = (uint64_t)(c.M / d.bm) * (c.N / d.bn), k_tiles = c.K / 64;
-    const uint64_t units = tiles * k_tiles, g = (uint64_t)cus;
-    // a run of at least four K tiles (less is not worth two launches) and of at most a tile's K extent
-    if (tiles >= g || units < 4 * g || (units + g - 1) / g > k_tiles) {
-        return 0;
+    const uint64_t tiles = (uint64_t)(c.M / d.bm) * (c.N / d.bn);
+    if (tiles == 0 || tiles > 0x7fffffffull) {
+        return false;
     }
-    return (uint32_t)g;
+    sk.g = (uint32_t)cus * (uint32_t)row->per_cu;
+    sk.r = (uint32_t)(tiles % sk.g);
+    sk.full_tiles = (uint32_t)(tiles - sk.r);
+    sk.k_tiles = c.K / 64;
+    sk.bm = d.bm;
+    sk.bn = d.bn;
+    if (sk.r == 0) {
+        return false;  // whole rounds only: nothing to stream
+    }
+    sk.splits = sk.g / sk.r;
+    sk.lefts = sk.g - sk.r * sk.splits;
+    const uint32_t even_run = (uint32_t)((uint64_t)sk.r * sk.k_tiles / sk.g);  // K tiles per workgroup, rounded down
+    sk.main_k = sk.lefts ? sk.splits * even_run : sk.k_tiles;
+    // a run of at least four K tiles (less is not worth a launch of its own and a summing pass)
+    return sk.main_k / sk.splits >= 4;
 }
 
-static size_t stream_k_bytes(int tile, uint32_t K, uint32_t workgroups)
+static GemmArgs::StreamKShape stream_k_shape(const StreamKLayout& sk)
 {
-    TileDims d;
-    tile_dims(tile, K, d);
-    return (size_t)2 * workgroups * d.bm * d.bn * 4;
+    return GemmArgs::StreamKShape{sk.full_tiles, sk.r, sk.splits, sk.main_k};
 }
 
-// Estimated run time of a stream-K plan in microseconds (constants as in plan_cost).
-static double stream_k_cost(const Canonical& c, int tile, uint32_t workgroups)
+// Estimated run time of a stream-K call in microseconds (constants as in plan_cost).
+static double stream_k_cost(const Canonical& c, int tile, const StreamKLayout& sk)
 {
-    TileDims d;
-    tile_dims(tile, c.K, d);
-    // (one workgroup per CU here)
     const TileRow& row = *tile_row(tile);
-    const double us_per_k64 = row.alone_k64, fixed_us = row.alone_us;
-    const double tiles = (double)(c.M / d.bm) * (c.N / d.bn), k_tiles = c.K / 64;
-    const double run = __builtin_ceil(tiles * k_tiles / workgroups);
-    const double tile_bytes = 4.0 * d.bm * d.bn, c_bytes = 4.0 * c.M * c.N;
-    // most workgroups store two parts (the second epilogue also waits for the first one's stores); then one pass reads
-    // every part and writes C
-    const double second_part_us = 9.0 * tile_bytes / 262144.0;
-    // Workgroups that run side by side sit at different K offsets and share no panel: every K tile of A and B rows is
-    // fetched once per workgroup, at the 6.2 TB/s the fabric delivered when this was measured.
-    const double fetch_us = tiles * k_tiles * (d.bm + d.bn) * 64.0 * 2.0 / 6.2e6;
-    const double loop_us = run * us_per_k64 > fetch_us ? run * us_per_k64 : fetch_us;
-    const double total = loop_us + fixed_us + second_part_us + 4.0 + ((workgroups + tiles) * tile_bytes + c_bytes) / 4.0e6;
-    return total * (1.0 + 1e-3);
+    const double tile_bytes = 4.0 * sk.bm * sk.bn, area = tile_bytes / 262144.0;
+    double total = 0.0;
+    if (sk.full_tiles > 0) {
+        // the whole rounds, as a plain launch of so many rounds is priced, and the gap between two launches
+        total += (double)(sk.full_tiles / sk.g) * (sk.k_tiles * row.us_k64 + row.fixed_us) + 3.0;
+    }
+    // The stream-K launch: every workgroup of the main partitions walks main_len K tiles in step with its
+    // neighbours (priced like split K); a leftover workgroup walks as many, in up to left_parts pieces, each with its
+    // own ring fill and tile store (7 us per 256 x 256 tile when a round of them ends together, 2 us of ring fill).
+    const double longest = sk.main_len() > sk.left_len() ? sk.main_len() : sk.left_len();
+    const double extra_parts = sk.left_parts() > 1 ? sk.left_parts() - 1.0 : 0.0;
+    // The leftover workgroups sit at unrelated K offsets and share no panel: every K tile of theirs is fetched once per
+    // workgroup, through the fabric, at the 3.3 to 3.8 TB/s measured when they are many (1536 x 2816 x 65536: 124 of 256
+    // workgroups of 256x128 tiles, 883 us; 160 of 512 of 192x128, 705 us).  With few of them the matrix cores set the pace.
+    const double left_fetch_us = (double)sk.lefts * sk.left_len() * (sk.bm + sk.bn) * 128.0 / 3.5e6;
+    const double loop_us = longest * row.alone_k64 > left_fetch_us ? longest * row.alone_k64 : left_fetch_us;
+    total += loop_us + row.alone_us + extra_parts * (7.0 * area + 2.0);
+    // then one pass reads every part and writes the tail tiles of C (2.5 us + 6 TB/s, as for summed K partitions)
+    total += 2.5 + ((double)sk.slots() + sk.r) * tile_bytes / 6.0e6;
+    // streaming floor, as in plan_cost: every byte of A, B and C crosses HBM at least once
+    const double M = (double)c.M, N = (double)c.N, K = (double)c.K;
+    const double hbm_us = (2.0 * (M * K + N * K) + 4.0 * M * N) / 5.0e6;
+    return (total > hbm_us ? total : hbm_us) * (1.0 + 1e-3);
 }
 
 // Estimated run time of a plan in microseconds.  One workgroup per CU for every tile (the rings fill the LDS).
@@ -424,18 +466,19 @@ static bool search_plan(const Canonical& c, int k_mode, int tile, size_t partial
         if (tile == MI_TILE_AUTO && !planner_considers(tl, c.K)) {
             continue;  // (a caller can still force it)
         }
-        // Stream-K only when asked for.  Measured on the deep-K shapes it is meant for (1024 x 2816 x 49152: 358 us
-        // against 246 us for five summed partitions): workgroups that run side by side sit at different K offsets
-        // of neighbouring tiles and share no panel, so every A and B byte is fetched once per workgroup and the launch
-        // runs at what the fabric delivers (6 TB/s), not at what the matrix cores take.
-        if (k_mode == MI_K_STREAM) {
-            const uint32_t wgs = stream_k_workgroups(c, tl, cus);
-            if (wgs > 0 && stream_k_bytes(tl, c.K, wgs) <= partial_space) {
-                const double cost = stream_k_cost(c, tl, wgs);
-                if (!found || cost < best) {
+        // Stream-K when asked for, or when the planner may choose and the workspace holds the parts.
+        // (Not by itself when an operand is larger than the memory-side cache: such a launch is a DRAM stream, priced
+        // by plan_cost with its read-once builds, which stream-K has none of.)
+        if (k_mode == MI_K_STREAM || (k_mode == MI_K_AUTO && partial_space > 0 && beyond_cache(c) == 0)) {
+            StreamKLayout sk;
+            if (stream_k_layout(c, tl, cus, sk) && sk.bytes() <= partial_space) {
+                const double cost = stream_k_cost(c, tl, sk);
+                // (left to itself the planner takes it only when it is priced clearly ahead: 3 %)
+                const double rank = k_mode == MI_K_AUTO ? cost * 1.03 : cost;
+                if (!found || rank < best) {
                     found = true;
-                    best = cost;
-                    plan = {tl, MI_K_STREAM, 1, wgs, cost};
+                    best = rank;
+                    plan = {tl, MI_K_STREAM, 1, sk.g, cost};
                 }
             }
         }
@@ -611,6 +654,24 @@ static Peel plan_peeled(const Canonical& c, int cus, double whole_cost_us)
     return best;
 }
 
+// The planner's own stream-K plan against the best plan that needs no workspace, peeled: a ragged or round-and-a-bit
+// problem may do better as an output-stationary launch plus strips than as whole rounds plus a streamed tail
+// (4096 x 4352 x 8192: 222 us peeled, 232 us streamed).  Replaces `plan` when the peeled estimate is the lower one.
+static void prefer_peeling_to_stream_k(const Canonical& c, int k_mode, int tile, Plan& plan)
+{
+    if (k_mode != MI_K_AUTO || tile != MI_TILE_AUTO || plan.k_mode != MI_K_STREAM) {
+        return;
+    }
+    Plan alt;
+    if (!make_plan(c, MI_K_OUTPUT_STATIONARY, tile, 0, alt)) {
+        return;
+    }
+    const Peel peel = plan_peeled(c, device_compute_units(), alt.cost_us);
+    if (peel.on && peel.cost_us < plan.cost_us) {
+        plan = alt;
+    }
+}
+
 __global__ __launch_bounds__(256) void zero_fill_kernel(float* dst, size_t n)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
@@ -675,49 +736,62 @@ static int reduce_partials(const float* partials, const Canonical& c, uint32_t s
     return MI_OK;
 }
 
-// Stream-K second pass: C tile t = sum, in workgroup order, of the parts that the workgroups whose runs overlap tile t
-// stored (see gemm_tn_kernel, STREAM).  One block per 8 rows of a tile; 16-byte accesses throughout.
+// Stream-K second pass: tail tile t of C = its main partitions' parts (slots t * S ... t * S + S - 1), then the parts
+// of the leftover workgroups whose runs overlap the tile's leftover K tiles (slot r * S + j + t for workgroup j), added
+// in that order (see gemm_tn_kernel, STREAM).  One block per 8 rows of a tile; 16-byte accesses throughout.
 __global__ __launch_bounds__(256) void stream_k_sum_kernel(const float* parts, float* c, uint32_t ldc, uint32_t bm, uint32_t bn,
                                                            uint32_t k_tiles, uint32_t workgroups, GemmArgs raster)
 {
     const uint32_t chunks = bm / 8;
     const uint32_t t = blockIdx.x / chunks, row0 = (blockIdx.x % chunks) * 8;
-    const uint64_t units = (uint64_t)raster.tiles_m * raster.tiles_n * k_tiles, g = workgroups;
-    const uint64_t first = (uint64_t)t * k_tiles, last = first + k_tiles - 1;  // this tile's run units
-    // workgroup l owns units [l * units / g, (l + 1) * units / g): the owner of unit x is ((x + 1) * g - 1) / units
-    const uint32_t l_first = (uint32_t)(((first + 1) * g - 1) / units), l_last = (uint32_t)(((last + 1) * g - 1) / units);
+    const uint32_t r = raster.sk.tiles, splits = raster.sk.splits, kr = k_tiles - raster.sk.main_k;
+    const uint32_t lefts = workgroups - r * splits;
+    // leftover workgroup j owns the leftover pairs [j * units / lefts, (j + 1) * units / lefts); tile t's are
+    // [t * kr, (t + 1) * kr)
+    const uint64_t units = (uint64_t)r * kr, first = (uint64_t)t * kr, last = first + kr;
+    uint32_t j_lo = 0, j_hi = 0;  // workgroups [j_lo, j_hi) overlap the tile
+    if (lefts) {
+        j_lo = (uint32_t)(first * lefts / units);
+        j_lo = j_lo ? j_lo - 1 : 0;
+        while (j_lo < lefts && (j_lo + 1) * units / lefts <= first) {
+            ++j_lo;
+        }
+        j_hi = j_lo;
+        while (j_hi < lefts && j_hi * units / lefts < last) {
+            ++j_hi;
+        }
+    }
     uint32_t tm, tn;
-    raster_tile(raster, t, tm, tn);
+    raster_tile(raster, raster.sk.first_tile + t, tm, tn);
     const uint32_t quads = bn / 4;
+    const size_t tile_elems = (size_t)bm * bn;
     for (uint32_t idx = threadIdx.x; idx < 8 * quads; idx += blockDim.x) {
         const uint32_t row = row0 + idx / quads, col = (idx % quads) * 4;
+        const size_t at = (size_t)row * bn + col;
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t l = l_first; l <= l_last; ++l) {
-            const uint64_t begin = l * units / g, end = (l + 1) * units / g;
-            if (end <= first || begin > last) {
-                continue;  // (cannot happen; keeps a rounding slip from reading a part that was never written)
+        for (uint32_t sp = 0; sp < splits; ++sp) {
+            acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts + (size_t)(t * splits + sp) * tile_elems + at));
+        }
+        for (uint32_t j = j_lo; j < j_hi; ++j) {
+            if ((uint64_t)j * units / lefts == (uint64_t)(j + 1) * units / lefts) {
+                continue;  // (an empty run stores nothing)
             }
-            const uint32_t part = begin / k_tiles == t ? 0u : 1u;
-            const float* src = parts + ((size_t)(2 * l + part) * bm + row) * bn + col;
-            acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src));
+            acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts + (size_t)(r * splits + j + t) * tile_elems + at));
         }
         *reinterpret_cast<f32x4*>(c + (size_t)(tm * bm + row) * ldc + (size_t)tn * bn + col) = acc;
     }
 }
 
-static int stream_k_sum(const float* parts, const Canonical& c, const Plan& plan, hipStream_t stream)
+static int stream_k_sum(const float* parts, const Canonical& c, const StreamKLayout& sk, hipStream_t stream)
 {
-    TileDims d;
-    if (!tile_dims(plan.tile, c.K, d)) {
-        return MI_ERR_BAD_ARGUMENT;
-    }
     GemmArgs raster{};
-    raster.tiles_m = c.M / d.bm;
-    raster.tiles_n = c.N / d.bn;
+    raster.tiles_m = c.M / sk.bm;
+    raster.tiles_n = c.N / sk.bn;
     raster.group_m = GROUP_M;
-    const uint32_t blocks = raster.tiles_m * raster.tiles_n * (d.bm / 8);
-    hipLaunchKernelGGL(stream_k_sum_kernel, dim3(blocks), dim3(256), 0, stream, parts, c.c, c.N, d.bm, d.bn, c.K / 64,
-                       plan.workgroups, raster);
+    raster.sk = stream_k_shape(sk);
+    const uint32_t blocks = sk.r * (sk.bm / 8);
+    hipLaunchKernelGGL(stream_k_sum_kernel, dim3(blocks), dim3(256), 0, stream, parts, c.c, c.ldc ? c.ldc : c.N, sk.bm, sk.bn,
+                       sk.k_tiles, sk.g, raster);
     MI_CHECK_LAUNCH();
     return MI_OK;
 }
@@ -933,6 +1007,9 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         p.c.launched_workgroups = timeline->out_workgroups;
     }
     const Canonical& c = p.c;
+    if (batch == nullptr && timeline == nullptr) {
+        prefer_peeling_to_stream_k(c, k_mode, tile, plan);
+    }
     if (tile == MI_TILE_AUTO && plan.k_mode == MI_K_OUTPUT_STATIONARY && batch == nullptr && timeline == nullptr) {
         const Peel peel = plan_peeled(c, device_compute_units(), plan.cost_us);
         if (peel.on) {
@@ -959,11 +1036,25 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         }
     }
     if (plan.k_mode == MI_K_STREAM) {
+        StreamKLayout sk;
+        if (!stream_k_layout(c, plan.tile, device_compute_units(), sk) || sk.g != plan.workgroups) {
+            return MI_ERR_UNSUPPORTED;
+        }
+        if (sk.full_tiles > 0) {
+            // the whole rounds of tiles: output stationary, stored straight into C
+            Canonical head = c;
+            head.first_tiles_only = sk.full_tiles;
+            const Plan head_plan{plan.tile, MI_K_OUTPUT_STATIONARY, 1, 0, 0.0};
+            if (const int st = launch_tile(t->ab_dtype, head, head_plan, stream)) {
+                return st;
+            }
+        }
         Canonical k = c;
         k.c = (float*)((char*)workspace + partial_off);
-        k.stream_k_workgroups = plan.workgroups;
+        k.stream_k_workgroups = sk.g;
+        k.sk = stream_k_shape(sk);
         const int st = launch_tile(t->ab_dtype, k, plan, stream);
-        return st || attributes_only ? st : stream_k_sum(k.c, c, plan, stream);
+        return st || attributes_only ? st : stream_k_sum(k.c, c, sk, stream);
     }
     if (plan.k_mode == MI_K_SPLIT_REDUCE) {
         // partition s of problem l stores its copy of C at partials[l][s]; the sum then writes the caller's C
@@ -1058,6 +1149,7 @@ static int describe_plan(const mi_gemm_tensors* t, int k_mode, int tile, size_t 
         used = (size_t)snprintf(out, out_size, "re-pack %s%s%s, then ", p.repack_a ? "A" : "", p.repack_a && p.repack_b ? " and " : "",
                                 p.repack_b ? "B" : "");
     }
+    prefer_peeling_to_stream_k(p.c, k_mode, tile, plan);
     if (tile == MI_TILE_AUTO && plan.k_mode == MI_K_OUTPUT_STATIONARY) {
         const Peel peel = plan_peeled(p.c, device_compute_units(), plan.cost_us);
         if (peel.on) {
@@ -1267,19 +1359,23 @@ int mi_matmul_mfma_workspace_bytes_for(const mi_gemm_tensors* t, int k_mode, int
     if (!make_plan(p.c, k_mode, tile, SIZE_MAX, plan)) {
         return MI_ERR_UNSUPPORTED;
     }
+    prefer_peeling_to_stream_k(p.c, k_mode, tile, plan);
     const size_t with_partials = round_up(p.ws_bytes, 256) + partial_bytes(p.c, plan.k_splits);
     *out_preferred = plan.k_mode == MI_K_SPLIT_REDUCE ? with_partials : p.ws_bytes;
     *out_required = p.ws_bytes;
     if (plan.k_mode == MI_K_STREAM) {
-        *out_preferred = round_up(p.ws_bytes, 256) + stream_k_bytes(plan.tile, p.c.K, plan.workgroups);
+        const int cus = device_compute_units();
+        StreamKLayout sk;
+        if (!stream_k_layout(p.c, plan.tile, cus, sk)) {
+            return MI_ERR_UNSUPPORTED;
+        }
+        *out_preferred = round_up(p.ws_bytes, 256) + sk.bytes();
         if (k_mode == MI_K_STREAM) {
-            // the forced mode runs with whatever holds the parts of the smallest tile that can be streamed
+            // the forced mode runs with whatever holds the parts of the tile that needs the least room
             size_t least = SIZE_MAX;
-            const int cus = device_compute_units();
             for (int tl = tile == MI_TILE_AUTO ? 1 : tile; tl <= (tile == MI_TILE_AUTO ? MI_TILE_COUNT_ - 1 : tile); ++tl) {
-                const uint32_t wgs = stream_k_workgroups(p.c, tl, cus);
-                if (wgs > 0 && stream_k_bytes(tl, p.c.K, wgs) < least) {
-                    least = stream_k_bytes(tl, p.c.K, wgs);
+                if (stream_k_layout(p.c, tl, cus, sk) && sk.bytes() < least) {
+                    least = sk.bytes();
                 }
             }
             *out_required = round_up(p.ws_bytes, 256) + least;

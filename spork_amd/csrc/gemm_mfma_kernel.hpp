@@ -59,6 +59,14 @@ struct GemmArgs {
     // 0: every K partition adds into the one C (the ATOMIC build).  Otherwise partition s stores its partial tile at
     // c + s * c_split_bytes with plain stores and a later pass sums the partitions.
     uint64_t c_split_bytes;
+    // Stream-K launches (the STREAM build) only, see StreamKShape: the tail tiles are raster tiles sk.first_tile ...
+    // sk.first_tile + sk.tiles - 1 of the tile grid above; `c` is then the parts buffer.
+    struct StreamKShape {
+        uint32_t first_tile;  // raster index of the first tile this launch works on
+        uint32_t tiles;       // r: how many tiles (fewer than workgroups)
+        uint32_t splits;      // S = workgroups / tiles: main partitions per tile, all tiles' partition s walked in step
+        uint32_t main_k;      // Km: K tiles of every tile that the main partitions cover ([s*Km/S, (s+1)*Km/S) each)
+    } sk;
     // Diagnostic timeline (null in normal use): workgroup g writes stamp i to timeline[(g * timeline_slots + i) * 2]
     // (the 100 MHz constant clock) and [.. + 1] (the core clock counter): kernel entry, then per work item the point where
     // K tile 0 has landed, the end of its K loop and the end of its epilogue issue, then the point where all of the
@@ -152,6 +160,19 @@ __device__ __forceinline__ void dma_buffer_to_lds_16B(__amdgpu_buffer_rsrc_t rsr
                                                       lds_char* lds_dst)
 {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds_dst, 16, voffset, soffset, 0, NONTEMPORAL ? 2 : 0);
+}
+
+// After a store of more than 8 bytes per lane the hardware needs two more instruction slots before the registers that
+// held its data may be written again.  The compiler knows the rule for ordinary vector instructions but not for the
+// moves between accumulation registers that it builds the next store's data with (seen in the ISA: the first register
+// of a store's quad overwritten by the very next instruction; on the GPU: one dword of a 16-byte store wrong, rarely,
+// when the store sat in the queue behind another workgroup's).  So every 16-byte store is followed by the two slots,
+// fenced so that nothing is scheduled into them.
+__device__ __forceinline__ void after_wide_store()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // Buffer descriptor over [base, base + bytes): raw (stride 0) addressing, 32-bit data format (dword 3 = 0x00020000).
@@ -316,13 +337,20 @@ __device__ __forceinline__ void map_work(const GemmArgs& p, uint32_t pid, uint32
 // stores outside C are dropped the same way.  Costs a few vector ALU operations per DMA and per store instruction, so
 // shapes that divide evenly use the EDGE = false build.  (Role of the predicated loads/stores of
 // gemm_baseline.cu:46,62,93 and of TMA out-of-bounds fill plus the bounds-checked store gemm_sm90.cu:654-668.)
-// STREAM (stream-K, the role of gemm_sm90.cu's stream_k modes): the (tile, K tile) pairs of the problem, tile-major in
-// raster order, are dealt in equal contiguous runs to the workgroups of a grid no larger than the chip, so every CU
-// works the same number of K tiles whatever the tile count.  The host guarantees that a run is no longer than one
-// tile's K extent: it covers the end of one tile and the start of the next at most, and the workgroup walks these
-// (at most two) parts one after the other.  Part `s` of logical workgroup `l` is stored as a dense BM x BN tile
-// (ldc = BN) at c + (2 * l + s) * BM * BN floats; a second kernel sums the parts of each tile into C.  Whole tiles
-// only (no EDGE), plain stores (no ATOMIC), one problem.
+// STREAM (stream-K, the role of gemm_sm90.cu's stream_k modes, gemm/gemm_sm90.cu:1004-1095): a launch of g workgroups
+// (one per CU) over r < g output tiles - the tiles that do not fill a round of CUs; full rounds run the plain build, as
+// the reference keeps them output stationary - with every workgroup given the same number of K tiles, r * KT / g.  A
+// contiguous run per workgroup over the (tile, K tile) pairs (the reference's dealing) puts workgroups that run side
+// by side at unrelated K offsets: on a chip with eight private L2s no two of them then read the same panel at the
+// same time and every byte of A and B is fetched once per workgroup.  So the dealing here keeps what makes split K
+// fast: S = g / r main partitions per tile, each Km / S K tiles long, and all r workgroups of partition s walk the
+// same K range in step (neighbouring tiles share their A and B panels through the L2); the K tiles [Km, KT) that are
+// left of every tile, r * (KT - Km) pairs, go in equal contiguous runs to the g - r * S workgroups that are left, each
+// of which then works on the leftovers of one or more tiles, one part after the other.  Every part is stored as a dense
+// BM x BN tile (ldc = BN) in the parts buffer: main partition s of tile t in slot t * S + s, the part of leftover
+// workgroup j on tile t in slot r * S + j + t (a run's parts and a tile's parts are consecutive in j and t, so j + t
+// names each once); a second kernel sums each tile's parts, in slot order, into C.  Whole tiles only (no EDGE), plain
+// stores (no ATOMIC), one problem.
 //
 // ONCE (whole tiles only): 1 = every byte of A, 2 = every byte of B is read by exactly one workgroup of
 // the launch (the problem is one tile wide in the other dimension) and the operand is larger than the memory-side
@@ -350,7 +378,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t wm = w / WN, wn = w % WN;
-    const uint32_t n_items = p.tiles_m * p.tiles_n * p.k_splits * p.batches;
+    const uint32_t n_items = gridDim.x;  // (all items of the problem, or its first whole rounds of tiles: see launch_cfg)
     const uint32_t kt_total = (p.K + BK - 1) / BK;
     constexpr uint32_t OOB = 0x80000000u;  // buffer offset that no descriptor below covers: loads give 0, stores drop
 
@@ -390,29 +418,55 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
         return it;
     };
-    // Stream-K: this workgroup's run of (tile, K tile) pairs is [run_begin, run_end) in units of K tiles
-    uint32_t n_parts = 1, run_tile = 0, stream_slot = 0;
-    uint64_t run_begin = 0, run_end = 0;
+    // Stream-K: this workgroup is main partition sk_split of tail tile sk_tile, or leftover workgroup sk_left with the
+    // run [sk_cur, sk_end) of the leftover (tile, K tile) pairs, walked one part (one tile's share) at a time.
+    uint32_t sk_tile = 0, sk_split = 0, sk_left = 0, sk_kr = 0;
+    uint64_t sk_cur = 0, sk_end = 0;
+    bool sk_main = false;
     if constexpr (STREAM) {
         const uint32_t l = logical_workgroup(blockIdx.x, gridDim.x);
-        const uint64_t units = (uint64_t)p.tiles_m * p.tiles_n * kt_total;
-        run_begin = l * units / gridDim.x;
-        run_end = (l + 1) * units / gridDim.x;
-        run_tile = (uint32_t)(run_begin / kt_total);
-        n_parts = run_end == run_begin ? 0u : run_end > (uint64_t)(run_tile + 1) * kt_total ? 2u : 1u;
-        stream_slot = 2u * l;
+        const uint32_t mains = p.sk.tiles * p.sk.splits;
+        sk_kr = kt_total - p.sk.main_k;
+        if (l < mains) {
+            // partition-major: the tiles of one partition are consecutive workgroups (and share panels in one L2)
+            sk_main = true;
+            sk_split = l / p.sk.tiles;
+            sk_tile = l % p.sk.tiles;
+            sk_cur = 0;
+            sk_end = 1;  // one part
+        }
+        else {
+            sk_left = l - mains;
+            const uint64_t units = (uint64_t)p.sk.tiles * sk_kr, lefts = gridDim.x - mains;
+            sk_cur = sk_left * units / lefts;
+            sk_end = (sk_left + 1) * units / lefts;
+        }
     }
-    auto make_part = [&](uint32_t part) {
+    auto make_part = [&]() {
         Item it;
-        const uint32_t tile = run_tile + part;
-        const uint64_t tile_first = (uint64_t)tile * kt_total;
-        const uint32_t kt_begin = part == 0 ? (uint32_t)(run_begin - tile_first) : 0u;
-        const uint32_t kt_end = run_end - tile_first < kt_total ? (uint32_t)(run_end - tile_first) : kt_total;
-        raster_tile(p, tile, it.tm, it.tn);
+        uint32_t tile, kt_begin, kt_end, slot;
+        if (sk_main) {
+            tile = sk_tile;
+            kt_begin = (uint32_t)((uint64_t)sk_split * p.sk.main_k / p.sk.splits);
+            kt_end = (uint32_t)((uint64_t)(sk_split + 1) * p.sk.main_k / p.sk.splits);
+            slot = sk_tile * p.sk.splits + sk_split;
+            sk_cur = sk_end;
+        }
+        else {
+            tile = (uint32_t)(sk_cur / sk_kr);
+            const uint32_t in_tile = (uint32_t)(sk_cur % sk_kr);
+            const uint64_t left_in_run = sk_end - sk_cur;
+            const uint32_t len = left_in_run < sk_kr - in_tile ? (uint32_t)left_in_run : sk_kr - in_tile;
+            kt_begin = p.sk.main_k + in_tile;
+            kt_end = kt_begin + len;
+            slot = p.sk.tiles * p.sk.splits + sk_left + tile;
+            sk_cur += len;
+        }
+        raster_tile(p, p.sk.first_tile + tile, it.tm, it.tn);
         it.KT = kt_end - kt_begin;
         it.a_base = (const char*)p.a + ((size_t)it.tm * BM * p.lda + (size_t)kt_begin * BK) * 2;
         it.b_base = (const char*)p.b + ((size_t)it.tn * BN * p.ldb + (size_t)kt_begin * BK) * 2;
-        it.c_tile = p.c + (size_t)(stream_slot + part) * (BM * BN);
+        it.c_tile = p.c + (size_t)slot * (BM * BN);
         it.m_rem = BM;
         it.n_rem = BN;
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
@@ -460,7 +514,9 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     // element of some K tile of this item's panels), or the one after it (NEXT = 1): the descriptors advance by one
     // K tile per iteration (two scalar adds) and the DMA itself needs no address arithmetic.  (The instruction's
     // immediate offset cannot name the next K tile: an LDS DMA adds it to the LDS address as well.)
-    auto issue_dma = [&](auto jc, auto immc, const char* ka, const char* kb, uint32_t dst_a, uint32_t dst_b) {
+    // `kla` / `klb` (range-checked build only): K elements that exist from the descriptor's K tile on.
+    auto issue_dma = [&](auto jc, auto immc, const char* ka, const char* kb, int32_t kla, int32_t klb, uint32_t dst_a,
+                         uint32_t dst_b) {
         constexpr int j = jc.value;
         constexpr int NEXT = immc.value;
         constexpr bool is_a = j < A_DMA;
@@ -479,8 +535,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             // the row part moves into the (range-checked) vector offset; a lane whose row or K chunk does not exist
             // asks for offset OOB instead
             const int32_t rows_left = is_a ? it.m_rem - jj * (NWAVES * RPI) : it.n_rem - (int32_t)Cfg::template b_row<PERM>(jj);
-            const int32_t k_done = (int32_t)((is_a ? ka - it.a_base : kb - it.b_base) / 2) + NEXT * BK;
-            const int32_t k_left = it.k_rem - k_done;
+            const int32_t k_left = (is_a ? kla : klb) - NEXT * BK;
             const bool exists = (int32_t)(is_a ? lrow : lrow_b) < rows_left && (int32_t)(lchunk * 8u) < k_left;
             const uint32_t voff = (is_a ? voff_a + jj * a_jstride : voff_b + Cfg::template b_row<PERM>(jj) * ldb2);
             dma_buffer_to_lds_16B(make_rsrc(is_a ? ka : kb, OOB), exists ? voff : OOB, NEXT * (BK * 2), dst);
@@ -536,13 +591,16 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         }
     };
 
-    for (uint32_t part = 0; part < n_parts; ++part) {
+    for (bool first_part = true; first_part || (STREAM && sk_cur < sk_end); first_part = false) {
     if constexpr (STREAM) {
-        if (part > 0) {
+        if (sk_cur >= sk_end) {
+            break;  // (a leftover workgroup whose run is empty)
+        }
+        if (!first_part) {
             // every wave has drained its fragment reads of the previous part (lgkmcnt(0) below): the ring may be refilled
             asm volatile("s_barrier" ::: "memory");
         }
-        cur = make_part(part);
+        cur = make_part();
     }
     // ---- prologue: start filling the ring, wait for tile 0, fetch its first fragments
     {
@@ -551,10 +609,11 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         for (int t = 0; t < PF; ++t) {
             if ((uint32_t)t < cur.KT) {
                 const char* const ka = cur.a_base + t * (BK * 2), * const kb = cur.b_base + t * (BK * 2);
-                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, ring_a(pos), ring_b(pos)); });
+                const int32_t kl = cur.k_rem - t * BK;
+                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
                 if (t < DIST_B) {
                     static_for<A_DMA, LPW>(
-                        [&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, ring_a(pos), ring_b(pos)); });
+                        [&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
                 }
             }
             pos = ring_next(pos);
@@ -597,6 +656,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         // refill begun in iteration kt fetches the K tile after it, BK * 2 bytes on)
         const char* ka = cur.a_base + (DIST_A - 1) * (BK * 2);
         const char* kb = cur.b_base + (DIST_B - 1) * (BK * 2);
+        int32_t kla = cur.k_rem - (DIST_A - 1) * BK, klb = cur.k_rem - (DIST_B - 1) * BK;  // K elements from there on
         // One K tile.  `steady` (compile time): every refill certainly happens, so the hot loop carries no branches;
         // otherwise (first and last PF iterations) they are decided at run time.
         auto k_tile = [&](auto steady, uint32_t kt) __attribute__((always_inline)) {
@@ -673,12 +733,12 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                             constexpr int j = Cfg::dma_index(dma_lo + dc.value);
                             if constexpr (last) {
                                 if (j < A_DMA ? ra_on : rb_on) {
-                                    issue_dma(IntC<j>{}, IntC<1>{}, ka, kb, ra_dst, rb_dst);
+                                    issue_dma(IntC<j>{}, IntC<1>{}, ka, kb, kla, klb, ra_dst, rb_dst);
                                 }
                             }
                             else {
                                 if (j < A_DMA ? pa_on : pb_on) {
-                                    issue_dma(IntC<j>{}, IntC<0>{}, ka, kb, pa_dst, pb_dst);
+                                    issue_dma(IntC<j>{}, IntC<0>{}, ka, kb, kla, klb, pa_dst, pb_dst);
                                 }
                             }
                         }
@@ -699,6 +759,8 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             }
             ka += BK * 2;
             kb += BK * 2;
+            kla -= BK;
+            klb -= BK;
         };
         {
             uint32_t kt = 0;
@@ -780,6 +842,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                                 const u32x4 bits = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
                                                     __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
                                 __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_c, voff, soff, NT);
+                                after_wide_store();
                             }
                         }
                     }
@@ -823,6 +886,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                                     const u32x4 bits = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
                                                         __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
                                     __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_c, inside ? voff + soff : OOB, 0u, NT);
+                                    after_wide_store();
                                 }
                             }
                         }

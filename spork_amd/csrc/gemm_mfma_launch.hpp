@@ -62,8 +62,13 @@ struct Canonical {
     // K partitions: 0 = they meet in C through atomics; otherwise partition s writes its own copy of C at
     // c + s * c_split_bytes (see GemmArgs::c_split_bytes)
     uint64_t c_split_bytes = 0;
-    // stream-K: `c` is the parts buffer (see gemm_tn_kernel) and this is the grid, at most one workgroup per CU
+    // stream-K: `c` is the parts buffer (see gemm_tn_kernel, STREAM), this is the grid (one workgroup per CU) and `sk`
+    // the way the tail tiles' K tiles are dealt to it
     uint32_t stream_k_workgroups = 0;
+    GemmArgs::StreamKShape sk{};
+    // a plain launch over the first `first_tiles_only` tiles of the raster order only (0: all tiles): the whole rounds
+    // of a problem whose last tiles run as a stream-K launch
+    uint32_t first_tiles_only = 0;
     // 1: A, 2: B is read once by the launch and too large to stay cached (see gemm_tn_kernel, ONCE); the launcher
     // ignores it where no such build exists
     int read_once = 0;
@@ -135,17 +140,28 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
     if ((uint64_t)args.k_tiles_per_split * (k_splits - 1) >= k_tiles) {
         return MI_ERR_UNSUPPORTED;
     }
-    const uint64_t items = (uint64_t)args.tiles_m * args.tiles_n * k_splits * c.batches;
+    uint64_t items = (uint64_t)args.tiles_m * args.tiles_n * k_splits * c.batches;
     if (items == 0 || items > 0x7fffffffull) {
         return MI_ERR_UNSUPPORTED;
     }
+    if (c.first_tiles_only > 0) {
+        if (k_splits != 1 || c.batches != 1 || c.first_tiles_only > items) {
+            return MI_ERR_UNSUPPORTED;
+        }
+        items = c.first_tiles_only;
+    }
     const bool stream_k = c.stream_k_workgroups > 0;
+    args.sk = c.sk;
     if (stream_k) {
-        // whole tiles, one problem, one run of K tiles per workgroup that is no longer than a tile's K extent (so that
-        // it touches two tiles at most) and not empty
-        const uint64_t units = (uint64_t)args.tiles_m * args.tiles_n * k_tiles;
-        const uint64_t g = c.stream_k_workgroups;
-        if (edge || k_splits != 1 || c.batches != 1 || Cfg::BK != 64 || g > units || (units + g - 1) / g > k_tiles) {
+        // whole tiles, one problem; the shape must be one that the host's stream_k_shape() makes: tail tiles inside the
+        // tile grid, fewer of them than workgroups, main partitions of at least one K tile each, leftover workgroups
+        // exactly when K tiles are left over
+        const uint64_t g = c.stream_k_workgroups, tiles = (uint64_t)args.tiles_m * args.tiles_n;
+        const GemmArgs::StreamKShape& sk = c.sk;
+        if (edge || k_splits != 1 || c.batches != 1 || Cfg::BK != 64 || sk.tiles == 0 || sk.tiles >= g ||
+            (uint64_t)sk.first_tile + sk.tiles > tiles || sk.splits != g / sk.tiles || sk.main_k > k_tiles ||
+            sk.main_k < sk.splits || ((g - (uint64_t)sk.tiles * sk.splits == 0) != (sk.main_k == k_tiles)) ||
+            c.first_tiles_only > 0) {
             return MI_ERR_UNSUPPORTED;
         }
         args.ldc = Cfg::BN;

@@ -183,7 +183,9 @@ def test_workspace_sum_of_k_partitions_sizes_and_validation():
     req, pref = S.matmul_mfma_workspace_bytes_for(t, S.K_SPLIT_REDUCE)
     assert pref == forced["k_splits"] * 1536 * 2304 * 4 and req == 2 * 1536 * 2304 * 4   # two partitions at least
     req, pref = S.matmul_mfma_workspace_bytes_for(t, S.K_AUTO)
-    assert req == 0 and pref > 0 and pref % (1536 * 2304 * 4) == 0
+    auto = S.matmul_mfma_describe(t, S.K_AUTO, S.TILE_AUTO, pref)
+    # (the planner's own choice with room is one of the two modes that use it: copies of C, or stream-K parts)
+    assert req == 0 and pref > 0 and ("stream k" in auto or pref % (1536 * 2304 * 4) == 0), auto
     # without a workspace the same call falls back to atomics; the plan query (no workspace) says so
     assert S.matmul_mfma_plan(t)["k_mode"] == "split k"
     # a problem that fills the chip unsplit prefers no workspace at all
@@ -202,17 +204,19 @@ def test_workspace_sum_of_k_partitions_sizes_and_validation():
     assert lib.mi_matmul_mfma_ws(C.byref(t), S.K_SPLIT_REDUCE, S.TILE_AUTO, 4096, 1 << 20, None) == 3
     assert lib.mi_matmul_mfma_ws(C.byref(t), S.K_SPLIT_REDUCE, S.TILE_AUTO, 4096, need - 1, None) == 3
     assert lib.mi_matmul_mfma_ws(C.byref(t), S.K_SPLIT_REDUCE, S.TILE_AUTO, 4100, need, None) == 3  # misaligned
-    # stream-K: forced only, whole tiles, fewer tiles than CUs; two parts of a tile per workgroup
+    # stream-K: whole tiles, a tile count that does not fill whole rounds of CUs.  44 tiles on 256 CUs (what the library
+    # assumes when no device is visible, and what an MI355X has): 5 main partitions per tile, 36 leftover workgroups,
+    # 44 * 5 + 36 + 44 - 1 parts
     t = _t(1024, 2816, 49152)
     sk = S.matmul_mfma_plan(t, S.K_STREAM, S.TILE_256x256)
     assert sk["k_mode"] == "stream k" and sk["k_splits"] == 1
-    cus = 256   # what the library assumes when no device is visible, and what an MI355X has
-    assert S.matmul_mfma_workspace_bytes_for(t, S.K_STREAM, S.TILE_256x256) == (2 * cus * 256 * 256 * 4,) * 2
+    assert S.matmul_mfma_workspace_bytes_for(t, S.K_STREAM, S.TILE_256x256) == (299 * 256 * 256 * 4,) * 2
     assert lib.mi_matmul_mfma(C.byref(t), S.K_STREAM, S.TILE_AUTO, None) == 3                 # needs the workspace
-    assert not S.matmul_mfma_supports(_t(8192, 8192, 8192), S.K_STREAM)                       # more tiles than CUs
+    assert not S.matmul_mfma_supports(_t(8192, 8192, 8192), S.K_STREAM)                       # whole rounds with every tile
+    assert S.matmul_mfma_supports(_t(8192 + 256, 8192, 8192), S.K_STREAM, S.TILE_256x256)     # four rounds and 32 tiles
     assert not S.matmul_mfma_supports(_t(1000, 2816, 49152), S.K_STREAM)                      # ragged M
     assert not S.matmul_mfma_supports(_t(1024, 2816, 49152 + 8), S.K_STREAM)                  # K not a multiple of 64
-    assert S.matmul_mfma_plan(t)["k_mode"] != "stream k"                                      # never chosen by itself
+    assert S.matmul_mfma_plan(t)["k_mode"] != "stream k"                                      # not without a workspace
     # argument checks of the query
     a, b = C.c_size_t(), C.c_size_t()
     assert lib.mi_matmul_mfma_workspace_bytes_for(None, S.K_AUTO, S.TILE_AUTO, C.byref(a), C.byref(b)) == 2

@@ -4,7 +4,9 @@ The kernel counts its own LDS reads with `s_waitcnt lgkmcnt(n)`, n > 0.  That co
 loads, which return out of order: one scalar load in flight next to the fragment reads would make the partial waits
 meaningless, silently.  So every scalar load must sit before the first fragment read, with a full wait in between.
 And the accumulators must stay in registers: a build whose plain (non-EDGE) kernels need scratch memory is a
-performance bug the tests would not otherwise see."""
+performance bug the tests would not otherwise see.  And no store of more than 8 bytes per lane may have its data
+registers written again within the next two instruction slots: the compiler does not insert those slots before the
+moves between accumulation registers, and the GPU then stores a half-overwritten value now and then."""
 import os
 import re
 import shutil
@@ -16,7 +18,8 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "spork_amd", "csrc")
-UNITS = ["gemm_mfma_inst_256x256.hip", "gemm_mfma_inst_64x128k32.hip"]  # the flagship tile and a 32x32x16 twin
+UNITS = ["gemm_mfma_inst_256x256.hip", "gemm_mfma_inst_64x128k32.hip",  # the flagship tile and a 32x32x16 twin
+         "gemm_mfma_inst_192x128.hip"]  # the tile of which two workgroups share a CU
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-munsafe-fp-atomics", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-S", "--cuda-device-only",
          "-Rpass-analysis=kernel-resource-usage"]
@@ -94,3 +97,37 @@ def test_plain_kernels_keep_everything_in_registers(compiled, unit):
             assert size == 0, (name, size)
         else:
             assert size <= 64, (name, size)
+
+
+def _registers(token):
+    m = re.match(r"([av])\[(\d+):(\d+)\]$", token)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.match(r"([av])(\d+)$", token)
+    return {(m.group(1), int(m.group(2)))} if m else set()
+
+
+@pytest.mark.parametrize("unit", UNITS)
+def test_wide_store_data_is_not_overwritten_in_the_next_two_slots(compiled, unit):
+    asm, _ = compiled[unit]
+    stores = 0
+    for name, lines in _kernels(asm):
+        code = [l.strip() for l in lines if l.startswith("\t") and not l.strip().startswith((";", "."))]
+        for i, line in enumerate(code):
+            if not re.match(r"(buffer|global)_store_dwordx[34]\b", line):
+                continue
+            stores += 1
+            data = _registers(line.split()[1].rstrip(","))
+            assert data, line
+            slots = 0
+            for nxt in code[i + 1:i + 4]:
+                op, _, rest = nxt.partition(" ")
+                if op == "s_nop":
+                    slots += int(rest.strip()) + 1
+                    continue
+                if slots >= 2:
+                    break
+                written = _registers(rest.split(",")[0].strip()) if op.startswith(("v_", "ds_read", "buffer_load", "global_load")) else set()
+                assert not (written & data), (name[-40:], line, nxt)
+                slots += 1
+    assert stores > 100 or "k32" in unit  # (the 32x32x16 twins store one dword per lane)
