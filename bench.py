@@ -3,11 +3,14 @@
 the C ABI of libmi_gemm.so on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3f16|c2|c4|c5|skinny] [--no-cpu] [--no-vendor]
+                    [--no-configs]
 
 A "step" is one GEMM launch on inputs already resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s over exactly
 K timed steps (host clock, synchronised on both sides), the per-launch roofline figure measured with HIP events on
 the launch stream (mean of the inter-quartile samples, the reference's statistic: gemm/gemm_test.cu:394-404), and the
-reference CPU GEMM (docs/nyc25.py:16-55) timed on a bounded sample of the same workload on this host's cores.
+reference CPU GEMM (docs/nyc25.py:16-55) timed on a bounded sample of the same workload on this host's cores (all of
+them, and one thread).  With the headline workload the line also carries a `configs` object: the other BASELINE
+configurations (fp16 4096^3, 16384x128x8192, 2048x2048x65536) measured the same way with fewer launches.
 PyTorch only provides device memory and the stream.
 """
 from __future__ import annotations
@@ -28,8 +31,11 @@ SETTLE_MS = 40.0      # untimed launches before the warm-up steps, see main()
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, KiB per dispatch,
 # scaled by the factor a plain copy kernel of known size reads on the same counters); summaries in profiles/.
-MEASURED_TRAFFIC_BYTES = {"c3": 1.882e9,      # profiles/gemm_tn_256x256_bf16_8192_pmc.md
-                          "skinny": 5.329e8}  # profiles/gemm_tn_256x128_read_once_bf16_256x8192x28672_kernel_stats_and_pmc.md
+MEASURED_TRAFFIC_BYTES = {"c3": 1.882e9, "skinny": 5.329e8}
+# ... and where each figure was recorded (rocprofv3 runs of this same command, not something measured in this run)
+TRAFFIC_SOURCE = {"c3": "profiles/gemm_tn_256x256_bf16_8192_pmc.md",
+                  "skinny": "profiles/gemm_tn_256x128_read_once_bf16_256x8192x28672_kernel_stats_and_pmc.md"}
+OTHER_CONFIGS = ("c2", "c4", "c5")  # the other BASELINE configurations that need a GPU, reported beside the headline
 
 WORKLOADS = {
     # name: (M, N, K, dtype, data_code, param_fn, description)
@@ -54,6 +60,7 @@ def main() -> int:
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the hipBLASLt comparator leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other BASELINE configurations (headline workload only)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the workload the CPU baseline computes (0 = auto)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy so that a rocprofv3 --pmc run of this command "
@@ -82,118 +89,13 @@ def main() -> int:
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    M, N, K, dtype_name, code, param_fn, desc = WORKLOADS[args.workload]
-    dtype = S.BF16 if dtype_name == "bf16" else S.F16
-    param = param_fn(K)
-    seed_a, seed_b = 20010106, 19980724  # the reference generator's constants (gemm/gemm_test.cu:76,87)
-
-    a = torch.empty((M, K), dtype=torch.int16, device="cuda")
-    b = torch.empty((N, K), dtype=torch.int16, device="cuda")
-    c = torch.empty((M, N), dtype=torch.float32, device="cuda")
-    c_check = torch.empty((M, N), dtype=torch.float32, device="cuda")
-    S.init_test_data(a.data_ptr(), M, K, code, False, dtype, param, seed_a, stream)
-    S.init_test_data(b.data_ptr(), N, K, code, True, dtype, param, seed_b, stream)
-    c.view(torch.uint8).fill_(0x7D)  # poison, gemm/gemm_test.cu:244-247
-    t = S.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), dtype, 0, 1, 0)
-    plan = S.matmul_mfma_plan(t)
-    # Deep-K workloads: with the workspace the library prefers, K partitions are summed from copies of C instead of
-    # through atomics.  Allocated once, outside the timed region; 0 bytes (and the plain entry point) for the rest.
-    _, ws_bytes = S.matmul_mfma_workspace_bytes_for(t)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
-    if ws is not None:
-        plan = S.matmul_mfma_plan(t, S.K_SPLIT_REDUCE)  # what K_AUTO picks when it is given that room
-
-        def launch():
-            S.matmul_mfma_ws(t, ws.data_ptr(), ws_bytes, S.K_AUTO, S.TILE_AUTO, stream)
-    else:
-        def launch():
-            S.matmul_mfma(t, S.K_AUTO, S.TILE_AUTO, stream)
-
-    # correctness of what is being timed: full-matrix compare against the on-device baseline kernel
-    launch()
-    tb = S.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c_check.data_ptr(), dtype, 0, 1, 0)
-    S.matmul_baseline(tb, stream)
-    res = torch.zeros(4, dtype=torch.int64, device="cuda")
-    S.compare_tensors(c_check.data_ptr(), c.data_ptr(), M, N, res.data_ptr(), stream)
-    torch.cuda.synchronize()
-    r = res.cpu().numpy().view("uint64")
-    import numpy as np
-
-    max_diff = float(np.array([r[1]]).view(np.float64)[0])
-    max_ref = float(np.array([r[2]]).view(np.float64)[0])
-    max_rel_err_vs_device_baseline = max_diff / max_ref if max_ref > 0 else float("inf")
-
-    if args.calibrate_copy:
-        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)  # 1 GiB
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-
-    # Settle the clocks first: measured on MI355X, after an idle spell the same launch runs 4 to 20 % slower for 25 to
-    # 30 ms before it reaches its steady rate, and a small --warmup / --steps would be timed inside that window.
-    settle_start = torch.cuda.Event(enable_timing=True)
-    settle_now = torch.cuda.Event(enable_timing=True)
-    settle_start.record()
-    settle_launches = 0
-    while settle_launches < 4096:
-        for _ in range(8):
-            launch()
-        settle_launches += 8
-        settle_now.record()
-        settle_now.synchronize()
-        if settle_start.elapsed_time(settle_now) >= SETTLE_MS:
-            break
-
-    for _ in range(args.warmup):
-        launch()
-    torch.cuda.synchronize()
-
-    # HIP events between launches, on the stream the kernel is launched on
-    events = []
-    for _ in range(args.steps + 1):
-        e = C.c_void_p()
-        S.capi.check(L.mi_rt_event_create(C.byref(e)), "event create")
-        events.append(e)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    L.mi_rt_event_record(events[0], stream)
-    for i in range(args.steps):
-        launch()
-        L.mi_rt_event_record(events[i + 1], stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    per_launch_ms = []
-    for i in range(args.steps):
-        ms = C.c_float()
-        S.capi.check(L.mi_rt_event_elapsed_ms(C.byref(ms), events[i], events[i + 1]), "event elapsed")
-        per_launch_ms.append(ms.value)
-    for e in events:
-        L.mi_rt_event_destroy(e)
-
-    flops = 2.0 * M * N * K
-    alg_bytes = 2.0 * (M * K + N * K) + 4.0 * M * N
-    total_s = t1 - t0
-    ms_per_step = total_s * 1e3 / args.steps
-    value = flops * args.steps / total_s * 1e-12
-    srt = sorted(per_launch_ms)
-    n = len(srt)
-    iqr = srt[n // 4: n // 4 + (n + 1) // 2]
-    launch_ms = sum(iqr) / len(iqr)  # gemm/gemm_test.cu:394-404
-    achieved = flops / (launch_ms * 1e-3) * 1e-12
-    ai = flops / alg_bytes
-    hbm_bound = ai * PEAK_HBM_GBS * 1e-3 < PEAK_TFLOPS  # TFLOP/s reachable at HBM peak
-    if hbm_bound:
-        ach_gbs = alg_bytes / (launch_ms * 1e-3) * 1e-9
-        roofline = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": round(ach_gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
-    else:
-        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
-    roofline.update({"kernel": f"gemm_tn_kernel tile {plan['tile']}, {plan['k_mode']}, k_splits {plan['k_splits']}",
-                     "launches": S.matmul_mfma_describe(t, workspace_bytes=ws_bytes),
-                     "launch_ms": round(launch_ms, 5), "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes})
+    m = measure(S, L, stream, args.workload, args.steps, args.warmup, SETTLE_MS, args.calibrate_copy)
+    M, N, K, dtype_name, dtype, code, param = m["M"], m["N"], m["K"], m["dtype_name"], m["dtype"], m["code"], m["param"]
+    desc, plan, flops, value, ms_per_step = m["desc"], m["plan"], m["flops"], m["value"], m["ms_per_step"]
+    roofline, achieved, settle_launches = m["roofline"], m["achieved"], m["settle_launches"]
+    max_rel_err_vs_device_baseline = m["max_rel_err_vs_device_baseline"]
+    a, b, c, t = m["a"], m["b"], m["c"], m["t"]
+    seed_a, seed_b = SEED_A, SEED_B
 
     out = {
         "metric": "TFLOP/s (2*M*N*K / t) of the bf16/fp16 -> fp32 GEMM at M=N=K=8192, and max rel err" if args.workload in ("c3", "c3f16")
@@ -228,9 +130,164 @@ def main() -> int:
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M, N, K, dtype, code, param, seed_a, seed_b, c, args.cpu_rows, out)
+        # the single-thread leg: the reference CPU GEMM as its authors run it, on a smaller sample of rows
+        out["cpu_baseline_1t"] = cpu_baseline(M, N, K, dtype, code, param, seed_a, seed_b, c, 0, None, threads=1, seconds=15.0)
+
+    if args.workload == "c3" and not args.no_configs:
+        # the other BASELINE configurations, one after the other on the same device: fewer launches, same protocol
+        del a, b, c, t, m
+        import torch
+
+        torch.cuda.empty_cache()
+        out["configs"] = {}
+        for name in OTHER_CONFIGS:
+            try:
+                r = measure(S, L, stream, name, 20, 5, 30.0)
+                out["configs"][name] = {
+                    "workload": r["desc"], "launch_ms": round(r["launch_ms"], 5),
+                    "tflops": round(r["flops"] / (r["launch_ms"] * 1e-3) * 1e-12, 1),
+                    "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac")},
+                    "max_rel_err": r["max_rel_err_vs_device_baseline"], "plan": r["roofline"]["launches"], "steps": 20}
+            except Exception as e:  # a side measurement must never take the benchmark line down
+                out["configs"][name] = {"error": str(e)[:200]}
+            r = None
+            torch.cuda.empty_cache()
 
     print(json.dumps(out), flush=True)
     return 0
+
+
+SEED_A, SEED_B = 20010106, 19980724  # the reference generator's constants (gemm/gemm_test.cu:76,87)
+
+
+def measure(S, L, stream, workload, steps, warmup, settle_ms, calibrate_copy=False) -> dict:
+    """One workload: seeded operands generated on the device, the planner's launch checked over the whole matrix against
+    the on-device baseline kernel, `settle_ms` of untimed launches, `warmup` more, then exactly `steps` timed ones."""
+    import torch
+
+    M, N, K, dtype_name, code, param_fn, desc = WORKLOADS[workload]
+    dtype = S.BF16 if dtype_name == "bf16" else S.F16
+    param = param_fn(K)
+    seed_a, seed_b = SEED_A, SEED_B
+
+    a = torch.empty((M, K), dtype=torch.int16, device="cuda")
+    b = torch.empty((N, K), dtype=torch.int16, device="cuda")
+    c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    c_check = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    S.init_test_data(a.data_ptr(), M, K, code, False, dtype, param, seed_a, stream)
+    S.init_test_data(b.data_ptr(), N, K, code, True, dtype, param, seed_b, stream)
+    c.view(torch.uint8).fill_(0x7D)  # poison, gemm/gemm_test.cu:244-247
+    t = S.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), dtype, 0, 1, 0)
+    plan = S.matmul_mfma_plan(t)
+    # Deep-K workloads: with the workspace the library prefers, K partitions are summed from copies of C instead of
+    # through atomics.  Allocated once, outside the timed region; 0 bytes (and the plain entry point) for the rest.
+    _, ws_bytes = S.matmul_mfma_workspace_bytes_for(t)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
+    if ws is not None:
+        # what K_AUTO picks when it is given that room: copies of C summed by a second kernel, or a stream-K tail
+        text = S.matmul_mfma_describe(t, workspace_bytes=ws_bytes)
+        if "stream k" in text:
+            plan = S.matmul_mfma_plan(t, S.K_STREAM)
+        elif "workspace sum" in text:
+            plan = S.matmul_mfma_plan(t, S.K_SPLIT_REDUCE)
+
+        def launch():
+            S.matmul_mfma_ws(t, ws.data_ptr(), ws_bytes, S.K_AUTO, S.TILE_AUTO, stream)
+    else:
+        def launch():
+            S.matmul_mfma(t, S.K_AUTO, S.TILE_AUTO, stream)
+
+    # correctness of what is being timed: full-matrix compare against the on-device baseline kernel
+    launch()
+    tb = S.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c_check.data_ptr(), dtype, 0, 1, 0)
+    S.matmul_baseline(tb, stream)
+    res = torch.zeros(4, dtype=torch.int64, device="cuda")
+    S.compare_tensors(c_check.data_ptr(), c.data_ptr(), M, N, res.data_ptr(), stream)
+    torch.cuda.synchronize()
+    r = res.cpu().numpy().view("uint64")
+    import numpy as np
+
+    max_diff = float(np.array([r[1]]).view(np.float64)[0])
+    max_ref = float(np.array([r[2]]).view(np.float64)[0])
+    max_rel_err_vs_device_baseline = max_diff / max_ref if max_ref > 0 else float("inf")
+
+    if calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    # Settle the clocks first: measured on MI355X, after an idle spell the same launch runs 4 to 20 % slower for 25 to
+    # 30 ms before it reaches its steady rate, and a small --warmup / --steps would be timed inside that window.
+    settle_start = torch.cuda.Event(enable_timing=True)
+    settle_now = torch.cuda.Event(enable_timing=True)
+    settle_start.record()
+    settle_launches = 0
+    while settle_launches < 4096:
+        for _ in range(8):
+            launch()
+        settle_launches += 8
+        settle_now.record()
+        settle_now.synchronize()
+        if settle_start.elapsed_time(settle_now) >= settle_ms:
+            break
+
+    for _ in range(warmup):
+        launch()
+    torch.cuda.synchronize()
+
+    # HIP events between launches, on the stream the kernel is launched on
+    events = []
+    for _ in range(steps + 1):
+        e = C.c_void_p()
+        S.capi.check(L.mi_rt_event_create(C.byref(e)), "event create")
+        events.append(e)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    L.mi_rt_event_record(events[0], stream)
+    for i in range(steps):
+        launch()
+        L.mi_rt_event_record(events[i + 1], stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    per_launch_ms = []
+    for i in range(steps):
+        ms = C.c_float()
+        S.capi.check(L.mi_rt_event_elapsed_ms(C.byref(ms), events[i], events[i + 1]), "event elapsed")
+        per_launch_ms.append(ms.value)
+    for e in events:
+        L.mi_rt_event_destroy(e)
+
+    flops = 2.0 * M * N * K
+    alg_bytes = 2.0 * (M * K + N * K) + 4.0 * M * N
+    total_s = t1 - t0
+    ms_per_step = total_s * 1e3 / steps
+    value = flops * steps / total_s * 1e-12
+    srt = sorted(per_launch_ms)
+    n = len(srt)
+    iqr = srt[n // 4: n // 4 + (n + 1) // 2]
+    launch_ms = sum(iqr) / len(iqr)  # gemm/gemm_test.cu:394-404
+    achieved = flops / (launch_ms * 1e-3) * 1e-12
+    ai = flops / alg_bytes
+    hbm_bound = ai * PEAK_HBM_GBS * 1e-3 < PEAK_TFLOPS  # TFLOP/s reachable at HBM peak
+    if hbm_bound:
+        ach_gbs = alg_bytes / (launch_ms * 1e-3) * 1e-9
+        roofline = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(ach_gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload)}
+    else:
+        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload)}
+    roofline.update({"kernel": f"gemm_tn_kernel tile {plan['tile']}, {plan['k_mode']}, k_splits {plan['k_splits']}",
+                     "launches": S.matmul_mfma_describe(t, workspace_bytes=ws_bytes),
+                     "launch_ms": round(launch_ms, 5), "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes})
+
+    roofline["traffic_source"] = TRAFFIC_SOURCE.get(workload)
+    return {"M": M, "N": N, "K": K, "dtype_name": dtype_name, "dtype": dtype, "code": code, "param": param, "desc": desc,
+            "plan": plan, "flops": flops, "value": value, "ms_per_step": ms_per_step, "roofline": roofline,
+            "achieved": achieved, "settle_launches": settle_launches, "launch_ms": launch_ms,
+            "max_rel_err_vs_device_baseline": max_rel_err_vs_device_baseline, "a": a, "b": b, "c": c, "t": t}
 
 
 def mfma_ceiling(S, L, a, dtype, stream):
@@ -345,17 +402,18 @@ def system_vendor_comparator(M, N, K, dtype_name, code, param) -> dict:
         return {"error": str(e)[:200]}
 
 
-def cpu_baseline(M, N, K, dtype, code, param, seed_a, seed_b, c_gpu, rows, out) -> dict:
+def cpu_baseline(M, N, K, dtype, code, param, seed_a, seed_b, c_gpu, rows, out, threads=0, seconds=15.0) -> dict:
     """The reference CPU GEMM (oracle port of nyc25_gemm_cpu) on the first `rows` rows of the same workload, OpenMP
     over m on this host's cores.  The oracle is only the thing timed and the checker here, never the product."""
     import numpy as np
 
     import oracle as O
 
-    threads = min(O.max_threads(), 16)  # the GPU box grants 16 cores per GPU whatever nproc says
+    if threads <= 0:
+        threads = min(O.max_threads(), 16)  # the GPU box grants 16 cores per GPU whatever nproc says
     if rows <= 0:
-        # aim for roughly 10-20 s of CPU work at ~1.5 GFLOP/s per thread for the scalar fp32 loop
-        rows = int(15.0 * 1.5e9 * threads / (2.0 * N * K))
+        # aim for roughly `seconds` of CPU work at ~1.5 GFLOP/s per thread for the scalar fp32 loop
+        rows = int(seconds * 1.5e9 * threads / (2.0 * N * K))
         rows = max(16, min(M, rows // 16 * 16))
     a = O.fill(rows, K, code, False, dtype, param, seed_a)  # rows 0..rows-1 of A (row-major: a prefix)
     b = O.fill(N, K, code, True, dtype, param, seed_b)
@@ -364,11 +422,13 @@ def cpu_baseline(M, N, K, dtype, code, param, seed_a, seed_b, c_gpu, rows, out) 
     dt = time.perf_counter() - t0
     c_dev = c_gpu[:rows].cpu().numpy()
     denom = float(np.abs(c_cpu).max())
-    out["max_rel_err_vs_cpu_sample"] = float(np.abs(c_dev.astype(np.float64) - c_cpu.astype(np.float64)).max() / denom)
-    return {"value": round(2.0 * rows * N * K / dt * 1e-12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    err = float(np.abs(c_dev.astype(np.float64) - c_cpu.astype(np.float64)).max() / denom)
+    if out is not None:
+        out["max_rel_err_vs_cpu_sample"] = err
+    return {"max_rel_err_of_gpu_vs_this_sample": err, "value": round(2.0 * rows * N * K / dt * 1e-12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "seconds": round(dt, 2),
             "sample": f"rows 0..{rows - 1} of M={M} (all N={N}, K={K}) of the same seeded workload; fp32 accumulate, "
-                      f"sequential k, OpenMP over m, gcc -O2"}
+                      f"sequential k, {'OpenMP over m' if threads > 1 else 'one thread'}, gcc -O2"}
 
 
 if __name__ == "__main__":

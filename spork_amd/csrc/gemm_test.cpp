@@ -250,9 +250,24 @@ int gemm_timeline(TimelineParams params, gpu_stream_t stream)
             gpu_check(st, "timeline launch");
         }
     }
-    // the clocks settle over a few milliseconds of load: warm up with plain launches, then report one stamped launch
-    for (uint32_t i = 0; i < params.warmup; ++i) {
-        gpu_check(mi_matmul_mfma(&abi, MI_K_AUTO, params.tile, stream), "warm-up launch");
+    // The clocks take 25 to 30 ms of load to settle: warm up with plain launches for at least `warmup` launches and
+    // 60 ms (a 100 us problem needs hundreds of them), then report one stamped launch.
+    {
+        void *w0 = nullptr, *w1 = nullptr;
+        gpu_check(mi_rt_event_create(&w0), "event create");
+        gpu_check(mi_rt_event_create(&w1), "event create");
+        gpu_check(mi_rt_event_record(w0, stream), "event record");
+        float ms = 0.0f;
+        for (uint32_t done = 0; done < 20000 && (done < params.warmup || ms < 60.0f);) {
+            for (uint32_t i = 0; i < 8; ++i, ++done) {
+                gpu_check(mi_matmul_mfma(&abi, MI_K_AUTO, params.tile, stream), "warm-up launch");
+            }
+            gpu_check(mi_rt_event_record(w1, stream), "event record");
+            gpu_check(mi_rt_event_synchronize(w1), "event sync");
+            gpu_check(mi_rt_event_elapsed_ms(&ms, w0, w1), "elapsed");
+        }
+        mi_rt_event_destroy(w0);
+        mi_rt_event_destroy(w1);
     }
     gpu_check(mi_rt_memset_async(d_stamps, 0, sizeof(uint64_t) * 2 * SLOTS * wgs, stream), "memset stamps");
     gpu_check(mi_matmul_mfma_timeline(&abi, MI_K_AUTO, params.tile, d_stamps, SLOTS, max_wg, &wgs, stream), "timeline launch");
