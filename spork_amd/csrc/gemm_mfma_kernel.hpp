@@ -54,6 +54,10 @@ struct GemmArgs {
     uint32_t k_splits;           // number of K partitions (1 = output stationary)
     uint32_t k_tiles_per_split;  // BK-tiles per partition (last one may be shorter)
     uint32_t group_m;            // tile-rows per raster group
+    // K rotation (0 = none; whole-tile builds only): the workgroups on XCD x walk their K range starting k_rotate * x
+    // K tiles in (modulo the range's length) and wrap around to its start, so that the XCDs are not all at the same
+    // K offset of their rows at the same time.
+    uint32_t k_rotate;
     uint32_t batches;            // independent problems of the same shape (>= 1)
     uint64_t a_batch_bytes, b_batch_bytes, c_batch_bytes;  // distance between consecutive problems
     // 0: every K partition adds into the one C (the ATOMIC build).  Otherwise partition s stores its partial tile at
@@ -398,6 +402,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
     // one work item: an output tile and a K range
     struct Item {
         uint32_t tm, tn, KT;
+        uint32_t rot;        // K tile of the range that the walk starts at (it wraps around to tile 0)
         const char* a_base;  // first row of the A panel, first K element of the range
         const char* b_base;
         float* c_tile;                // where element (0, 0) of this item's output tile goes
@@ -416,6 +421,8 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         it.m_rem = (int32_t)(p.M - it.tm * BM);
         it.n_rem = (int32_t)(p.N - it.tn * BN);
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
+        // (short ranges are not rotated: the walk's look-ahead must stay inside one lap)
+        it.rot = EDGE || it.KT < 16 ? 0u : ((blockIdx.x % NUM_XCD) * p.k_rotate) % it.KT;
         return it;
     };
     // Stream-K: this workgroup is main partition sk_split of tail tile sk_tile, or leftover workgroup sk_left with the
@@ -470,12 +477,18 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         it.m_rem = BM;
         it.n_rem = BN;
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
+        it.rot = 0;
         return it;
     };
     Item cur;
     if constexpr (!STREAM) {
         cur = make_item(blockIdx.x);
     }
+    // K tile of the item's range that step `step` of the walk works on (steps beyond the range are never fetched)
+    auto walk_tile = [](const Item& it, uint32_t step) {
+        const uint32_t at = it.rot + step;
+        return at >= it.KT ? at - it.KT : at;
+    };
 
     // ---- consumer addressing (LDS byte addresses inside slot 0)
     const uint32_t g = lane / MT;      // which 8-wide k group of the MFMA's K depth this lane feeds
@@ -497,48 +510,43 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
 
     // Scalar byte offsets of the rows that DMA instruction jj of wave 0 fetches (the per-instruction part of the
     // address): loop invariant, one SGPR each.
-    // ([0]: of the K tile the descriptor is based at, [1]: of the K tile after it)
-    uint32_t soff_a[2][A_DMA > 0 ? A_DMA : 1], soff_b[2][LPW - A_DMA > 0 ? LPW - A_DMA : 1];
+    uint32_t soff_a[A_DMA > 0 ? A_DMA : 1], soff_b[LPW - A_DMA > 0 ? LPW - A_DMA : 1];
 #pragma unroll
     for (int jj = 0; jj < A_DMA; ++jj) {
-        soff_a[0][jj] = jj * a_jstride;
-        soff_a[1][jj] = jj * a_jstride + BK * 2;
+        soff_a[jj] = jj * a_jstride;
     }
 #pragma unroll
     for (int jj = 0; jj < LPW - A_DMA; ++jj) {
-        soff_b[0][jj] = Cfg::template b_row<PERM>(jj) * ldb2;
-        soff_b[1][jj] = Cfg::template b_row<PERM>(jj) * ldb2 + BK * 2;
+        soff_b[jj] = Cfg::template b_row<PERM>(jj) * ldb2;
     }
     // DMA instruction j of this wave: for j < A_DMA rows of A into the LDS region at byte `dst_a`, else rows of B into
     // the region at `dst_b`.  The K tile is the one the buffer descriptors `ka` / `kb` are based at (the first K
-    // element of some K tile of this item's panels), or the one after it (NEXT = 1): the descriptors advance by one
-    // K tile per iteration (two scalar adds) and the DMA itself needs no address arithmetic.  (The instruction's
-    // immediate offset cannot name the next K tile: an LDS DMA adds it to the LDS address as well.)
+    // element of some K tile of this item's panels): the descriptors move on by one K tile per iteration, at the
+    // hand-off barrier (a few scalar operations), and the DMA itself needs no address arithmetic.
     // `kla` / `klb` (range-checked build only): K elements that exist from the descriptor's K tile on.
-    auto issue_dma = [&](auto jc, auto immc, const char* ka, const char* kb, int32_t kla, int32_t klb, uint32_t dst_a,
+    auto issue_dma = [&](auto jc, const char* ka, const char* kb, int32_t kla, int32_t klb, uint32_t dst_a,
                          uint32_t dst_b) {
         constexpr int j = jc.value;
-        constexpr int NEXT = immc.value;
         constexpr bool is_a = j < A_DMA;
         constexpr int jj = is_a ? j : j - A_DMA;
         const Item& it = cur;  // (captured by reference: the item lives for the whole kernel)
         lds_char* const dst = lds_w + (is_a ? dst_a : dst_b) + jj * (NWAVES * 1024);
         if constexpr (!EDGE) {
             if constexpr (is_a) {
-                dma_buffer_to_lds_16B<ONCE == 1>(make_rsrc(ka, BM * p.lda * 2u), voff_a, soff_a[NEXT][jj], dst);
+                dma_buffer_to_lds_16B<ONCE == 1>(make_rsrc(ka, BM * p.lda * 2u), voff_a, soff_a[jj], dst);
             }
             else {
-                dma_buffer_to_lds_16B<ONCE == 2>(make_rsrc(kb, BN * p.ldb * 2u), voff_b, soff_b[NEXT][jj], dst);
+                dma_buffer_to_lds_16B<ONCE == 2>(make_rsrc(kb, BN * p.ldb * 2u), voff_b, soff_b[jj], dst);
             }
         }
         else {
             // the row part moves into the (range-checked) vector offset; a lane whose row or K chunk does not exist
             // asks for offset OOB instead
             const int32_t rows_left = is_a ? it.m_rem - jj * (NWAVES * RPI) : it.n_rem - (int32_t)Cfg::template b_row<PERM>(jj);
-            const int32_t k_left = (is_a ? kla : klb) - NEXT * BK;
+            const int32_t k_left = is_a ? kla : klb;
             const bool exists = (int32_t)(is_a ? lrow : lrow_b) < rows_left && (int32_t)(lchunk * 8u) < k_left;
             const uint32_t voff = (is_a ? voff_a + jj * a_jstride : voff_b + Cfg::template b_row<PERM>(jj) * ldb2);
-            dma_buffer_to_lds_16B(make_rsrc(is_a ? ka : kb, OOB), exists ? voff : OOB, NEXT * (BK * 2), dst);
+            dma_buffer_to_lds_16B(make_rsrc(is_a ? ka : kb, OOB), exists ? voff : OOB, 0, dst);
         }
     };
     // fragment read i of a k-step: B fragments first, then A fragments (the order the MFMA rows need them)
@@ -608,12 +616,13 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
 #pragma unroll
         for (int t = 0; t < PF; ++t) {
             if ((uint32_t)t < cur.KT) {
-                const char* const ka = cur.a_base + t * (BK * 2), * const kb = cur.b_base + t * (BK * 2);
-                const int32_t kl = cur.k_rem - t * BK;
-                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
+                const uint32_t kt_of_t = walk_tile(cur, t);
+                const char* const ka = cur.a_base + (size_t)kt_of_t * (BK * 2);
+                const char* const kb = cur.b_base + (size_t)kt_of_t * (BK * 2);
+                const int32_t kl = cur.k_rem - t * BK;  // (range-checked build: never rotated)
+                static_for<0, A_DMA>([&](auto jc) { issue_dma(jc, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
                 if (t < DIST_B) {
-                    static_for<A_DMA, LPW>(
-                        [&](auto jc) { issue_dma(jc, IntC<0>{}, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
+                    static_for<A_DMA, LPW>([&](auto jc) { issue_dma(jc, ka, kb, kl, kl, ring_a(pos), ring_b(pos)); });
                 }
             }
             pos = ring_next(pos);
@@ -652,10 +661,13 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         for (int k = 0; k < PERIOD; ++k) {
             u[k] = (uint32_t)k * (SPLIT ? UNIT : (uint32_t)STAGE_BYTES);
         }
-        // K tile kt + DIST - 1 of this item's panels (the rest of the refill begun in iteration kt-1 fetches it; the
-        // refill begun in iteration kt fetches the K tile after it, BK * 2 bytes on)
-        const char* ka = cur.a_base + (DIST_A - 1) * (BK * 2);
-        const char* kb = cur.b_base + (DIST_B - 1) * (BK * 2);
+        // Step kt + DIST - 1 of the walk over this item's panels: the rest of the refill begun in iteration kt-1 fetches
+        // it.  At the hand-off barrier of iteration kt the descriptors move on to the next step (wrapping around at the
+        // end of the range when the walk is rotated), which the refill begun there fetches.
+        const char* ka = cur.a_base + (size_t)walk_tile(cur, DIST_A - 1) * (BK * 2);
+        const char* kb = cur.b_base + (size_t)walk_tile(cur, DIST_B - 1) * (BK * 2);
+        const char* const a_end = cur.a_base + (size_t)cur.KT * (BK * 2);
+        const char* const b_end = cur.b_base + (size_t)cur.KT * (BK * 2);
         int32_t kla = cur.k_rem - (DIST_A - 1) * BK, klb = cur.k_rem - (DIST_B - 1) * BK;  // K elements from there on
         // One K tile.  `steady` (compile time): every refill certainly happens, so the hot loop carries no branches;
         // otherwise (first and last PF iterations) they are decided at run time.
@@ -701,6 +713,16 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     else {
                         wait_vmcnt_then_barrier<0>();
                     }
+                    ka += BK * 2;
+                    kb += BK * 2;
+                    if constexpr (EDGE) {
+                        kla -= BK;
+                        klb -= BK;
+                    }
+                    else {
+                        ka = ka == a_end ? cur.a_base : ka;
+                        kb = kb == b_end ? cur.b_base : kb;
+                    }
                 }
                 else {
                     // B fragments and the first A fragment of this k-step; the other A fragments may still be in flight
@@ -733,12 +755,12 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                             constexpr int j = Cfg::dma_index(dma_lo + dc.value);
                             if constexpr (last) {
                                 if (j < A_DMA ? ra_on : rb_on) {
-                                    issue_dma(IntC<j>{}, IntC<1>{}, ka, kb, kla, klb, ra_dst, rb_dst);
+                                    issue_dma(IntC<j>{}, ka, kb, kla, klb, ra_dst, rb_dst);
                                 }
                             }
                             else {
                                 if (j < A_DMA ? pa_on : pb_on) {
-                                    issue_dma(IntC<j>{}, IntC<0>{}, ka, kb, kla, klb, pa_dst, pb_dst);
+                                    issue_dma(IntC<j>{}, ka, kb, kla, klb, pa_dst, pb_dst);
                                 }
                             }
                         }
@@ -757,10 +779,6 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             for (int k = 0; k < PERIOD; ++k) {
                 u[k] = turned[k];
             }
-            ka += BK * 2;
-            kb += BK * 2;
-            kla -= BK;
-            klb -= BK;
         };
         {
             uint32_t kt = 0;

@@ -85,6 +85,7 @@ struct Canonical {
 };
 
 constexpr uint32_t GROUP_M = 4;  // tile-rows per raster group (see map_work)
+constexpr uint32_t K_ROTATE_TILES = 37;  // K tiles between the starting points of consecutive XCDs' walks (see launch_cfg)
 
 template <int DTYPE, typename Cfg, bool ATOMIC, bool EDGE, bool STREAM = false, int ONCE = 0>
 int launch_kernel(const GemmArgs& args, uint32_t grid, hipStream_t stream, bool attributes_only)
@@ -129,6 +130,16 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
     const uint32_t k_tiles = (c.K + Cfg::BK - 1) / Cfg::BK;
     args.k_tiles_per_split = (k_tiles + k_splits - 1) / k_splits;
     args.group_m = GROUP_M;
+    // K partitions of rows whose stride is a large power of two (the dense layout of a deep power-of-two K) all sit at
+    // the same offset of their rows modulo that stride, and every row's bytes at one K offset map to the same few
+    // memory channels: when all XCDs walk K from the start of their partition the launch queues up on those channels
+    // (2048 x 2048 x 65536 in four partitions: 2660 core cycles per K tile against 2320 with rows padded by 128 B).
+    // Starting each XCD's walk 37 K tiles further into its partition spreads them: measured 0.97 of the run time on
+    // that problem, 0.88 on 2048 x 1024 x 65536 in eight partitions, 0.92 on 1024 x 1024 x 131072 in sixteen, within
+    // 1 % either way on other power-of-two strides; on strides that are not powers of two it can cost up to 6 %.
+    const uint64_t row_bytes = (uint64_t)c.lda * 2;
+    const bool aliasing_rows = c.lda == c.ldb && row_bytes >= 65536 && (row_bytes & (row_bytes - 1)) == 0;
+    args.k_rotate = (k_splits > 1 && !edge && aliasing_rows) ? K_ROTATE_TILES : 0;
     args.timeline = c.timeline;
     args.timeline_slots = c.timeline_slots;
     args.batches = c.batches;

@@ -240,6 +240,42 @@ def test_mfma_split_k_workspace_sum(gpu, oracle, dtype, tile, shape):
     assert H.rel_err(c.cpu().numpy(), runs[0].astype(np.float64)) < 1e-5
 
 
+ROTATED_WALK_CASES = [  # (tile name, M, N, K, forced partitions or 0 for the planner's)
+    ("TILE_256x256", 256, 256, 32768, 2),    # two workgroups, on XCD 0 (walk from the start) and XCD 1 (37 K tiles in)
+    ("TILE_128x128", 512, 512, 32768, 2),    # 32 workgroups: every XCD, the walks of XCD 7 start 3 tiles in (259 mod 256)
+    ("TILE_128x128", 512, 512, 32768, 0),
+    ("TILE_64x128", 128, 256, 65536, 0),
+    ("TILE_256x128", 256, 384, 32768, 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("case", ROTATED_WALK_CASES)
+def test_mfma_split_k_rotated_walk(gpu, oracle, dtype, case):
+    """Rows of a power-of-two length of 64 KB or more: the workgroups of XCD x walk their K partition from 37 * x K tiles
+    in and wrap around to its start.  Every K tile must still be used exactly once, whatever the partition length."""
+    tile_name, M, N, K, forced = case
+    tile = getattr(gpu, tile_name)
+    a, b = H.make_inputs(M, N, K, dtype, 3, 3, 0.5)
+    ref = oracle.gemm_f64(M, N, K, H.to_host_u16(a), H.to_host_u16(b), dtype)
+    c = H.poisoned_c(M, N)
+    t = H.tensors(M, N, K, a, b, c, dtype)
+    if forced:
+        need, _ = gpu.matmul_mfma_workspace_bytes_for(t, gpu.K_SPLIT_REDUCE, tile)
+        assert need == forced * M * N * 4
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        gpu.matmul_mfma_ws(t, ws.data_ptr(), need, gpu.K_SPLIT_REDUCE, tile, H.stream_handle())
+        k_tiles = K // 64 // forced
+    else:
+        plan = gpu.matmul_mfma_plan(t, gpu.K_SPLIT, tile)
+        assert plan["k_splits"] > 1
+        k_tiles = -(-(K // 64) // plan["k_splits"])
+        gpu.matmul_mfma(t, gpu.K_SPLIT, tile, H.stream_handle())
+    torch.cuda.synchronize()
+    assert k_tiles >= 16, "partitions this short are not rotated: the case no longer tests the wrap-around"
+    assert H.rel_err(c.cpu().numpy(), ref) < TOL
+
+
 STREAM_CASES = [  # (tile, bm, bn, tiles_m, tiles_n, K tiles): 4 to 5 K tiles per workgroup; leftover runs cross tiles
     # more tiles than CUs: whole rounds run output stationary, the rest is streamed (272 = 256 + 16 tiles with no
     # leftover workgroups; 280 = 256 + 24 with 16 of them; 552 = 2 * 256 + 40)
