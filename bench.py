@@ -31,9 +31,12 @@ SETTLE_MS = 40.0      # untimed launches before the warm-up steps, see main()
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, KiB per dispatch,
 # scaled by the factor a plain copy kernel of known size reads on the same counters); summaries in profiles/.
-MEASURED_TRAFFIC_BYTES = {"c3": 1.882e9, "skinny": 5.329e8}
+MEASURED_TRAFFIC_BYTES = {"c3": 1.880e9, "c2": 2.688e8, "c4": 2.953e8, "c5": 1.215e9, "skinny": 5.329e8}
 # ... and where each figure was recorded (rocprofv3 runs of this same command, not something measured in this run)
 TRAFFIC_SOURCE = {"c3": "profiles/gemm_tn_256x256_bf16_8192_pmc.md",
+                  "c2": "profiles/gemm_tn_256x256_f16_4096_kernel_stats_pmc_timeline.md",
+                  "c4": "profiles/gemm_tn_64x128_f16_16384x128x8192_kernel_stats_pmc_timeline.md",
+                  "c5": "profiles/gemm_split_k_workspace_sum_f16_2048x2048x65536_kernel_stats_pmc_timeline.md",
                   "skinny": "profiles/gemm_tn_256x128_read_once_bf16_256x8192x28672_kernel_stats_and_pmc.md"}
 OTHER_CONFIGS = ("c2", "c4", "c5")  # the other BASELINE configurations that need a GPU, reported beside the headline
 
@@ -146,7 +149,7 @@ def main() -> int:
                 out["configs"][name] = {
                     "workload": r["desc"], "launch_ms": round(r["launch_ms"], 5),
                     "tflops": round(r["flops"] / (r["launch_ms"] * 1e-3) * 1e-12, 1),
-                    "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac")},
+                    "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
                     "max_rel_err": r["max_rel_err_vs_device_baseline"], "plan": r["roofline"]["launches"], "steps": 20}
             except Exception as e:  # a side measurement must never take the benchmark line down
                 out["configs"][name] = {"error": str(e)[:200]}
