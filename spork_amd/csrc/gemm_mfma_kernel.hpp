@@ -147,6 +147,51 @@ __device__ __forceinline__ void touch(u32x4& x)
     asm volatile("" : "+v"(x));
 }
 
+// A scalar move / a scalar-plus-vector add that stays where it is written (the compiler would otherwise gather such
+// bookkeeping at the top of the loop, where it delays the first MFMAs of a K tile).
+__device__ __forceinline__ uint32_t pinned_move(uint32_t x)
+{
+    uint32_t r;
+    asm volatile("s_mov_b32 %0, %1" : "=s"(r) : "s"(x));
+    return r;
+}
+__device__ __forceinline__ uint32_t pinned_add(uint32_t s, uint32_t v)
+{
+    uint32_t r;
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(s), "v"(v));
+    return r;
+}
+
+// The DMA in two hand-placed halves, for loops that give every instruction an MFMA gap of its own: the LDS base goes
+// into M0 one gap ahead (the write needs a wait state before a DMA may use it, which the MFMA in between provides), the
+// DMA itself names a descriptor held in four scalar registers.  The compiler does not know that M0 is live between the
+// two: the loops that use them contain no other user of M0 (checked in the ISA by the code generation test).
+// (M0 is on the clobber list so that the compiler re-initialises it before any LDS DMA of its own that follows, e.g.
+// the ring fill of a stream-K workgroup's next part; clang remarks that M0 is a reserved register, which is the point.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma_set_lds_base(uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0" ::"s"(lds_addr) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <bool NONTEMPORAL>
+__device__ __forceinline__ void dma_issue_16B(u32x4 rsrc, uint32_t voffset, uint32_t soffset)
+{
+    if constexpr (NONTEMPORAL) {
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen nt lds" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+    }
+    else {
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+    }
+}
+// Descriptor words for [base, base + bytes), as make_rsrc builds them
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, uint32_t bytes)
+{
+    const uint64_t b = (uint64_t)(uintptr_t)base & 0xffffffffffffull;
+    return u32x4{(uint32_t)b, (uint32_t)(b >> 32), bytes, 0x00020000u};
+}
+
 // No instruction may be scheduled across this point.  (Device-only builtins are kept out of lambda bodies: the host
 // pass silently drops the kernel stub of a __global__ template whose lambdas name them.)
 __device__ __forceinline__ void sched_fence()
@@ -664,11 +709,44 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         // Step kt + DIST - 1 of the walk over this item's panels: the rest of the refill begun in iteration kt-1 fetches
         // it.  At the hand-off barrier of iteration kt the descriptors move on to the next step (wrapping around at the
         // end of the range when the walk is rotated), which the refill begun there fetches.
-        const char* ka = cur.a_base + (size_t)walk_tile(cur, DIST_A - 1) * (BK * 2);
-        const char* kb = cur.b_base + (size_t)walk_tile(cur, DIST_B - 1) * (BK * 2);
-        const char* const a_end = cur.a_base + (size_t)cur.KT * (BK * 2);
-        const char* const b_end = cur.b_base + (size_t)cur.KT * (BK * 2);
+        const char* const a_begin = cur.a_base, * const b_begin = cur.b_base;
+        const char* ka = a_begin + (size_t)walk_tile(cur, DIST_A - 1) * (BK * 2);
+        const char* kb = b_begin + (size_t)walk_tile(cur, DIST_B - 1) * (BK * 2);
+        const char* const a_end = a_begin + (size_t)cur.KT * (BK * 2);
+        const char* const b_end = b_begin + (size_t)cur.KT * (BK * 2);
         int32_t kla = cur.k_rem - (DIST_A - 1) * BK, klb = cur.k_rem - (DIST_B - 1) * BK;  // K elements from there on
+        // LDS addresses (per lane) that the fragment reads issued during the coming k-step start from: computed one
+        // k-step ahead, in MFMA gaps of their own, so that no k-step begins with a clump of address arithmetic
+        uint32_t rd_a = a_off[1 % KS] + u[0], rd_b = b_off[1 % KS] + u[SPLIT ? 1 : 0] + (SPLIT ? 0u : (uint32_t)Cfg::A_BYTES);
+        // The ring offsets are turned in place, one scalar move per MFMA gap at the end of a K tile's last k-step (after
+        // the last DMA that names an old offset), when that k-step has the gaps to spare.
+        constexpr int ROT_MOVES = PERIOD + 1;
+        constexpr int LAST_DMA_I = ((Cfg::DMA_PER_STEP - 1) * NMFMA) / Cfg::DMA_PER_STEP + 1;
+        constexpr int RD_I = (NR - 1) * RS + 2;  // first gap after the k-step's last fragment read
+        constexpr bool LATE = Cfg::LOOP_READS == NR && RD_I + 3 <= NMFMA - ROT_MOVES && LAST_DMA_I < NMFMA - ROT_MOVES;
+        uint32_t u_tmp = 0;
+        // Loops with gaps to spare also place their DMAs by hand (dma_set_lds_base / dma_issue_16B) and carry the two
+        // descriptors themselves (words 0 and 1 are the 48-bit base) instead of the pointers `ka` / `kb`.
+        // (every DMA then sits in an odd gap at least two gaps after the one before it, so that the gap ahead of it exists
+        // and lies behind the previous DMA)
+        constexpr bool ASM_DMA = LATE && !EDGE && (NMFMA / Cfg::DMA_PER_STEP) >= 2 && RS % 2 == 0;
+        u32x4 qa = make_rsrc_words(ka, BM * p.lda * 2u), qb = make_rsrc_words(kb, BN * p.ldb * 2u);
+        const uint64_t a_begin48 = (uint64_t)(uintptr_t)a_begin & 0xffffffffffffull, a_end48 = a_begin48 + (uint64_t)cur.KT * (BK * 2);
+        const uint64_t b_begin48 = (uint64_t)(uintptr_t)b_begin & 0xffffffffffffull, b_end48 = b_begin48 + (uint64_t)cur.KT * (BK * 2);
+        auto quad_step = [](u32x4& q) {
+            const uint64_t b = (((uint64_t)q.y << 32) | q.x) + BK * 2;
+            q.x = (uint32_t)b;
+            q.y = (uint32_t)(b >> 32);
+        };
+        auto quad_wrap = [](u32x4& q, uint64_t begin, uint64_t end) {
+            uint64_t b = ((uint64_t)q.y << 32) | q.x;
+            b = b == end ? begin : b;
+            q.x = (uint32_t)b;
+            q.y = (uint32_t)(b >> 32);
+        };
+        // ... and the descriptors move on in the last gaps of the k-step before the hand-off barrier (their old
+        // position is last named by that k-step's last DMA), not in the gap right behind the barrier.
+        constexpr bool EARLY_ADV = LATE && KS >= 2 && LAST_DMA_I < NMFMA - 5;
         // One K tile.  `steady` (compile time): every refill certainly happens, so the hot loop carries no branches;
         // otherwise (first and last PF iterations) they are decided at run time.
         auto k_tile = [&](auto steady, uint32_t kt) __attribute__((always_inline)) {
@@ -697,8 +775,15 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                 constexpr int dma_hi = dma_lo + Cfg::DMA_PER_STEP < LPW ? dma_lo + Cfg::DMA_PER_STEP : LPW;
                 constexpr int dma_n = dma_hi - dma_lo;
                 // source of the next k-step's fragments: same tile, or k-step 0 of the next tile
-                const uint32_t a_nx = last ? a_off[0] + a_nxt : a_off[(ks + 1) % KS] + a_cur;
-                const uint32_t b_nx = last ? b_off[0] + b_nxt : b_off[(ks + 1) % KS] + b_cur;
+                uint32_t a_nx, b_nx, a_nn = 0, b_nn = 0;
+                if constexpr (LATE) {
+                    a_nx = rd_a;
+                    b_nx = rd_b;
+                }
+                else {
+                    a_nx = last ? a_off[0] + a_nxt : a_off[(ks + 1) % KS] + a_cur;
+                    b_nx = last ? b_off[0] + b_nxt : b_off[(ks + 1) % KS] + b_cur;
+                }
                 if constexpr (last) {
                     // Every fragment of tile kt is now in registers and this wave's share of tile kt+1 has landed:
                     // after the barrier the regions of tile kt may be refilled and tile kt+1 may be read.  DMAs land
@@ -713,15 +798,17 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     else {
                         wait_vmcnt_then_barrier<0>();
                     }
-                    ka += BK * 2;
-                    kb += BK * 2;
-                    if constexpr (EDGE) {
-                        kla -= BK;
-                        klb -= BK;
-                    }
-                    else {
-                        ka = ka == a_end ? cur.a_base : ka;
-                        kb = kb == b_end ? cur.b_base : kb;
+                    if constexpr (!EARLY_ADV) {
+                        ka += BK * 2;
+                        kb += BK * 2;
+                        if constexpr (EDGE) {
+                            kla -= BK;
+                            klb -= BK;
+                        }
+                        else {
+                            ka = ka == a_end ? a_begin : ka;
+                            kb = kb == b_end ? b_begin : kb;
+                        }
                     }
                 }
                 else {
@@ -746,13 +833,98 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     }
                     acc[mi][ni] = mfma_tile<DTYPE>(fa[cu][mi], fb[cu][ni], acc[mi][ni]);
                     sched_fence();
+                    if constexpr (LATE && (i == RD_I || i == RD_I + 2)) {
+                        // read bases of the next k-step: fragments of k-step ks+2 of this tile, of k-step 0 of the next
+                        // tile (next k-step is this tile's last) or of k-step 1 of the next tile (this one is)
+                        constexpr int of = ks + 2 < KS ? ks + 2 : ks + 2 == KS ? 0 : 1;
+                        const uint32_t su = i == RD_I ? (ks + 2 < KS ? a_cur : a_nxt) : (ks + 2 < KS ? b_cur : b_nxt);
+                        if constexpr (i == RD_I) {
+                            a_nn = pinned_add(su, a_off[of]);
+                        }
+                        else {
+                            b_nn = pinned_add(su, b_off[of]);
+                        }
+                    }
+                    if constexpr (EARLY_ADV && ks == KS - 2 && i >= NMFMA - 5 && i < NMFMA - 1) {
+                        constexpr int m = i - (NMFMA - 5);
+                        if constexpr (ASM_DMA) {
+                            if constexpr (m == 0) {
+                                quad_step(qa);
+                            }
+                            else if constexpr (m == 1) {
+                                quad_wrap(qa, a_begin48, a_end48);
+                            }
+                            else if constexpr (m == 2) {
+                                quad_step(qb);
+                            }
+                            else {
+                                quad_wrap(qb, b_begin48, b_end48);
+                            }
+                        }
+                        else if constexpr (m == 0) {
+                            ka += BK * 2;
+                            if constexpr (EDGE) {
+                                kla -= BK;
+                            }
+                        }
+                        else if constexpr (m == 1) {
+                            if constexpr (!EDGE) {
+                                ka = ka == a_end ? a_begin : ka;
+                            }
+                        }
+                        else if constexpr (m == 2) {
+                            kb += BK * 2;
+                            if constexpr (EDGE) {
+                                klb -= BK;
+                            }
+                        }
+                        else {
+                            if constexpr (!EDGE) {
+                                kb = kb == b_end ? b_begin : kb;
+                            }
+                        }
+                    }
+                    if constexpr (LATE && last && i >= NMFMA - ROT_MOVES) {
+                        // move m of the rotation u[k] <- u[(k + STEP) % PERIOD], walked as one cycle from position 0
+                        constexpr int m = i - (NMFMA - ROT_MOVES);
+                        if constexpr (m == 0) {
+                            u_tmp = pinned_move(u[0]);
+                        }
+                        else if constexpr (m == PERIOD) {
+                            u[((PERIOD - 1) * STEP) % PERIOD] = pinned_move(u_tmp);
+                        }
+                        else {
+                            u[((m - 1) * STEP) % PERIOD] = pinned_move(u[(m * STEP) % PERIOD]);
+                        }
+                    }
                     if constexpr (i % RS == 0 && i / RS < NR) {
                         issue_read(IntC<i / RS>{}, IntC<nx>{}, a_nx, b_nx);
                     }
-                    // DMA d of this k-step goes after MFMA d*NMFMA/dma_n (evenly spaced)
+                    // DMA d of this k-step goes after MFMA d*NMFMA/dma_n (evenly spaced), one further on when the fragment
+                    // reads sit in the even gaps
                     static_for<0, dma_n>([&](auto dc) {
-                        if constexpr ((dc.value * NMFMA) / dma_n == i) {
-                            constexpr int j = Cfg::dma_index(dma_lo + dc.value);
+                        constexpr int slot = (dc.value * NMFMA) / dma_n + ((NMFMA / dma_n) >= 2 && RS % 2 == 0 ? 1 : 0);
+                        constexpr int j = Cfg::dma_index(dma_lo + dc.value);
+                        if constexpr (ASM_DMA) {
+                            constexpr bool is_a = j < A_DMA;
+                            constexpr int jj = is_a ? j : j - A_DMA;
+                            const uint32_t region = last ? (is_a ? ra_dst : rb_dst) : (is_a ? pa_dst : pb_dst);
+                            if constexpr (slot - 1 == i) {
+                                // LDS base of the DMA, a gap ahead of it
+                                dma_set_lds_base((uint32_t)(uintptr_t)(lds_w + region + jj * (NWAVES * 1024)));
+                            }
+                            if constexpr (slot == i) {
+                                if (last ? (is_a ? ra_on : rb_on) : (is_a ? pa_on : pb_on)) {
+                                    if constexpr (is_a) {
+                                        dma_issue_16B<ONCE == 1>(qa, voff_a, soff_a[jj]);
+                                    }
+                                    else {
+                                        dma_issue_16B<ONCE == 2>(qb, voff_b, soff_b[jj]);
+                                    }
+                                }
+                            }
+                        }
+                        else if constexpr (slot == i) {
                             if constexpr (last) {
                                 if (j < A_DMA ? ra_on : rb_on) {
                                     issue_dma(IntC<j>{}, ka, kb, kla, klb, ra_dst, rb_dst);
@@ -768,16 +940,22 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     sched_fence();
                 });
                 static_for<Cfg::LOOP_READS, NR>([&](auto ic) { issue_read(ic, IntC<nx>{}, a_nx, b_nx); });
+                if constexpr (LATE) {
+                    rd_a = a_nn;
+                    rd_b = b_nn;
+                }
             });
             // on to the next K tile: the ring turns by STEP positions
-            uint32_t turned[PERIOD];
+            if constexpr (!LATE) {
+                uint32_t turned[PERIOD];
 #pragma unroll
-            for (int k = 0; k < PERIOD; ++k) {
-                turned[k] = u[(k + STEP) % PERIOD];
-            }
+                for (int k = 0; k < PERIOD; ++k) {
+                    turned[k] = u[(k + STEP) % PERIOD];
+                }
 #pragma unroll
-            for (int k = 0; k < PERIOD; ++k) {
-                u[k] = turned[k];
+                for (int k = 0; k < PERIOD; ++k) {
+                    u[k] = turned[k];
+                }
             }
         };
         {
@@ -786,8 +964,13 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             for (; kt < KT && kt + 1 < (uint32_t)PF; ++kt) {
                 k_tile(IntC<0>{}, kt);
             }
-            for (; kt + PF < KT; ++kt) {
-                k_tile(IntC<1>{}, kt);
+            {
+                // (the steady iterations do not look at kt: a plain countdown)
+                const uint32_t n_steady = __builtin_amdgcn_readfirstlane(KT > kt + (uint32_t)PF ? KT - kt - (uint32_t)PF : 0u);
+                for (uint32_t n = n_steady; n != 0; --n) {
+                    k_tile(IntC<1>{}, 0u);
+                }
+                kt += n_steady;
             }
             for (; kt < KT; ++kt) {
                 k_tile(IntC<0>{}, kt);

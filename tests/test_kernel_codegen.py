@@ -131,3 +131,51 @@ def test_wide_store_data_is_not_overwritten_in_the_next_two_slots(compiled, unit
                 assert not (written & data), (name[-40:], line, nxt)
                 slots += 1
     assert stores > 100 or "k32" in unit  # (the 32x32x16 twins store one dword per lane)
+
+
+def _branch_free_loops(lines):
+    """Bodies of the loops (label ... backward branch to it) that contain no other branch: the steady K loops."""
+    labels = {m.group(1): i for i, l in enumerate(lines) if (m := re.match(r"(\.LBB\d+_\d+):", l))}
+    for i, l in enumerate(lines):
+        m = re.match(r"\s+s_cbranch_\w+ (\.LBB\d+_\d+)", l)
+        if m and labels.get(m.group(1), i) < i:
+            body = [x.strip() for x in lines[labels[m.group(1)] + 1:i] if x.startswith("\t") and not x.strip().startswith((";", "."))]
+            if not any(x.startswith(("s_cbranch", "s_branch")) for x in body):
+                yield body
+
+
+def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled):
+    """The K loop of the largest tile issues its DMAs through inline assembly: `s_mov_b32 m0, <LDS base>` in one MFMA gap,
+    the `buffer_load_dwordx4 ... lds` that reads M0 in the next.  The compiler does not know M0 is live in between, so
+    nothing else may write M0 there: in the steady loop of every whole-tile build each DMA must be preceded by exactly
+    one write of M0 since the DMA before it, that write must be the hand-placed move, and an MFMA (the wait state the
+    write needs) must lie between the two.  (The general iterations at either end of the K loop run the same source with
+    the DMAs under run-time flags; their branches make a linear reading of the listing meaningless.)"""
+    asm, _ = compiled["gemm_mfma_inst_256x256.hip"]
+    checked = 0
+    for name, lines in _kernels(asm):
+        if "Lb1ELb0ELi0EEEvNS_8GemmArgsE" in name:  # range-checked builds keep the compiler's own DMA
+            continue
+        loops = [b for b in _branch_free_loops(lines) if sum(x.startswith("v_mfma") for x in b) >= 64]
+        assert loops, name[-40:]
+        for body in loops:
+            # (the loop is a cycle: start reading at its first DMA so that the write ahead of it is seen at the end)
+            first = next(i for i, l in enumerate(body) if l.startswith("buffer_load_dwordx4"))
+            body = body[first + 1:] + body[:first + 1]
+            writes, mfma_since_write, dmas = [], 0, 0
+            for l in body:
+                op = l.split()[0]
+                if op.startswith("s_") and re.search(r"\bm0\b", l.split(",")[0]):
+                    writes.append(l)
+                    mfma_since_write = 0
+                elif op.startswith("v_mfma"):
+                    mfma_since_write += 1
+                elif op == "buffer_load_dwordx4":
+                    assert l.rstrip().endswith("lds"), l
+                    dmas += 1
+                    assert len(writes) == 1 and writes[0].startswith("s_mov_b32 m0, s"), (name[-40:], writes)
+                    assert mfma_since_write >= 1, name[-40:]
+                    writes = []
+            assert dmas == 16, (name[-40:], dmas)
+            checked += 1
+    assert checked >= 10
