@@ -163,16 +163,23 @@ __device__ __forceinline__ uint32_t pinned_add(uint32_t s, uint32_t v)
 }
 
 // The DMA in two hand-placed halves, for loops that give every instruction an MFMA gap of its own: the LDS base goes
-// into M0 one gap ahead (the write needs a wait state before a DMA may use it, which the MFMA in between provides), the
+// into M0 one gap ahead (base + a constant in one scalar add; the write needs a wait state before a DMA may use it,
+// which the MFMA in between provides), the
 // DMA itself names a descriptor held in four scalar registers.  The compiler does not know that M0 is live between the
 // two: the loops that use them contain no other user of M0 (checked in the ISA by the code generation test).
 // (M0 is on the clobber list so that the compiler re-initialises it before any LDS DMA of its own that follows, e.g.
 // the ring fill of a stream-K workgroup's next part; clang remarks that M0 is a reserved register, which is the point.)
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
+template <int IMM>
 __device__ __forceinline__ void dma_set_lds_base(uint32_t lds_addr)
 {
-    asm volatile("s_mov_b32 m0, %0" ::"s"(lds_addr) : "memory", "m0");
+    if constexpr (IMM == 0) {
+        asm volatile("s_mov_b32 m0, %0" ::"s"(lds_addr) : "memory", "m0");
+    }
+    else {
+        asm volatile("s_add_i32 m0, %0, %1" ::"s"(lds_addr), "n"(IMM) : "memory", "m0", "scc");
+    }
 }
 #pragma clang diagnostic pop
 template <bool NONTEMPORAL>
@@ -911,7 +918,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                             const uint32_t region = last ? (is_a ? ra_dst : rb_dst) : (is_a ? pa_dst : pb_dst);
                             if constexpr (slot - 1 == i) {
                                 // LDS base of the DMA, a gap ahead of it
-                                dma_set_lds_base((uint32_t)(uintptr_t)(lds_w + region + jj * (NWAVES * 1024)));
+                                dma_set_lds_base<jj * (NWAVES * 1024)>((uint32_t)(uintptr_t)(lds_w + region));
                             }
                             if constexpr (slot == i) {
                                 if (last ? (is_a ? ra_on : rb_on) : (is_a ? pa_on : pb_on)) {

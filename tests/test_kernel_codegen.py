@@ -146,7 +146,7 @@ def _branch_free_loops(lines):
 
 def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled):
     """The K loop of the largest tile issues its DMAs through inline assembly: `s_mov_b32 m0, <LDS base>` in one MFMA gap,
-    the `buffer_load_dwordx4 ... lds` that reads M0 in the next.  The compiler does not know M0 is live in between, so
+    the `buffer_load_dwordx4 ... lds` that reads M0 in the next (`s_add_i32 m0, <base>, <constant>` for all but the first).  The compiler does not know M0 is live in between, so
     nothing else may write M0 there: in the steady loop of every whole-tile build each DMA must be preceded by exactly
     one write of M0 since the DMA before it, that write must be the hand-placed move, and an MFMA (the wait state the
     write needs) must lie between the two.  (The general iterations at either end of the K loop run the same source with
@@ -173,7 +173,7 @@ def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled):
                 elif op == "buffer_load_dwordx4":
                     assert l.rstrip().endswith("lds"), l
                     dmas += 1
-                    assert len(writes) == 1 and writes[0].startswith("s_mov_b32 m0, s"), (name[-40:], writes)
+                    assert len(writes) == 1 and re.match(r"s_(mov_b32 m0, s\d+|add_i32 m0, s\d+, 0x[0-9a-f]+)$", writes[0]), (name[-40:], writes)
                     assert mfma_since_write >= 1, name[-40:]
                     writes = []
             assert dmas == 16, (name[-40:], dmas)
