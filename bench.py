@@ -31,7 +31,7 @@ SETTLE_MS = 40.0      # untimed launches before the warm-up steps, see main()
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, KiB per dispatch,
 # scaled by the factor a plain copy kernel of known size reads on the same counters); summaries in profiles/.
-MEASURED_TRAFFIC_BYTES = {"c3": 1.880e9, "c2": 2.688e8, "c4": 2.953e8, "c5": 1.215e9, "skinny": 5.329e8}
+MEASURED_TRAFFIC_BYTES = {"c3": 1.880e9, "c2": 2.687e8, "c4": 2.997e8, "c5": 1.224e9, "skinny": 5.329e8}
 # ... and where each figure was recorded (rocprofv3 runs of this same command, not something measured in this run)
 TRAFFIC_SOURCE = {"c3": "profiles/gemm_tn_256x256_bf16_8192_pmc.md",
                   "c2": "profiles/gemm_tn_256x256_f16_4096_kernel_stats_pmc_timeline.md",
