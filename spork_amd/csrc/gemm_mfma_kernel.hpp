@@ -208,7 +208,8 @@ __device__ __forceinline__ void sched_fence()
 
 // One wave-level DMA (`buffer_load_dwordx4 ... lds`): lane i copies 16 B from buffer byte (voffset_i + soffset) to
 // LDS byte (lds_dst + 16*i).  lds_dst is wave-uniform (it travels in M0), soffset is wave-uniform (an SGPR), so a
-// K-tile advance costs one scalar add and no vector ALU work; the per-lane offset is a single 32-bit VGPR.  Bytes
+// K-tile advance is scalar work on the descriptor's base and no vector ALU work; the per-lane offset is a single
+// 32-bit VGPR.  Bytes
 // past the descriptor's num_records read as zero.  Completion is tracked by vmcnt.  NONTEMPORAL sets the
 // instruction's `nt` bit: the line is marked for early eviction in the L2 and the memory-side cache.
 template <bool NONTEMPORAL = false>
