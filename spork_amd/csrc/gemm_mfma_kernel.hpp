@@ -727,17 +727,25 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         // k-step ahead, in MFMA gaps of their own, so that no k-step begins with a clump of address arithmetic
         uint32_t rd_a = a_off[1 % KS] + u[0], rd_b = b_off[1 % KS] + u[SPLIT ? 1 : 0] + (SPLIT ? 0u : (uint32_t)Cfg::A_BYTES);
         // The ring offsets are turned in place, one scalar move per MFMA gap at the end of a K tile's last k-step (after
-        // the last DMA that names an old offset), when that k-step has the gaps to spare.
+        // the last DMA that names an old offset), when a k-step has the gaps to spare (LATE: all tiles but the three
+        // smallest 64-deep ones and the 32-deep twins).
         constexpr int ROT_MOVES = PERIOD + 1;
-        constexpr int LAST_DMA_I = ((Cfg::DMA_PER_STEP - 1) * NMFMA) / Cfg::DMA_PER_STEP + 1;
         constexpr int RD_I = (NR - 1) * RS + 2;  // first gap after the k-step's last fragment read
-        constexpr bool LATE = Cfg::LOOP_READS == NR && RD_I + 3 <= NMFMA - ROT_MOVES && LAST_DMA_I < NMFMA - ROT_MOVES;
+        // DMA d of a k-step sits in gap d * DMA_STRIDE + 1: evenly over the k-step if that leaves the last gaps free for
+        // the moves below, else over the part of the k-step ahead of them
+        constexpr int DPS = Cfg::DMA_PER_STEP;
+        constexpr int TAIL_GAPS = ROT_MOVES > 5 ? ROT_MOVES : 5;  // ring moves (last k-step) / descriptor advance (the one before)
+        constexpr int EVEN_STRIDE = NMFMA / DPS;
+        constexpr int DMA_STRIDE = (DPS - 1) * EVEN_STRIDE + 1 < NMFMA - TAIL_GAPS ? EVEN_STRIDE : (NMFMA - TAIL_GAPS - 1) / DPS;
+        constexpr int LAST_DMA_I = (DPS - 1) * DMA_STRIDE + 1;
+        constexpr bool LATE = Cfg::LOOP_READS == NR && KS >= 2 && DMA_STRIDE >= 2 && RD_I + 3 <= NMFMA - ROT_MOVES &&
+                              LAST_DMA_I < NMFMA - TAIL_GAPS;
         uint32_t u_tmp = 0;
         // Loops with gaps to spare also place their DMAs by hand (dma_set_lds_base / dma_issue_16B) and carry the two
         // descriptors themselves (words 0 and 1 are the 48-bit base) instead of the pointers `ka` / `kb`.
-        // (every DMA then sits in an odd gap at least two gaps after the one before it, so that the gap ahead of it exists
-        // and lies behind the previous DMA)
-        constexpr bool ASM_DMA = LATE && !EDGE && (NMFMA / Cfg::DMA_PER_STEP) >= 2 && RS % 2 == 0;
+        // (every DMA sits at least two gaps after the one before it and not in gap 0, so that the gap ahead of it exists and
+        // lies behind the previous DMA)
+        constexpr bool ASM_DMA = LATE && !EDGE;
         u32x4 qa = make_rsrc_words(ka, BM * p.lda * 2u), qb = make_rsrc_words(kb, BN * p.ldb * 2u);
         const uint64_t a_begin48 = (uint64_t)(uintptr_t)a_begin & 0xffffffffffffull, a_end48 = a_begin48 + (uint64_t)cur.KT * (BK * 2);
         const uint64_t b_begin48 = (uint64_t)(uintptr_t)b_begin & 0xffffffffffffull, b_end48 = b_begin48 + (uint64_t)cur.KT * (BK * 2);
@@ -754,7 +762,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         };
         // ... and the descriptors move on in the last gaps of the k-step before the hand-off barrier (their old
         // position is last named by that k-step's last DMA), not in the gap right behind the barrier.
-        constexpr bool EARLY_ADV = LATE && KS >= 2 && LAST_DMA_I < NMFMA - 5;
+        constexpr bool EARLY_ADV = LATE;
         // One K tile.  `steady` (compile time): every refill certainly happens, so the hot loop carries no branches;
         // otherwise (first and last PF iterations) they are decided at run time.
         auto k_tile = [&](auto steady, uint32_t kt) __attribute__((always_inline)) {
@@ -908,10 +916,11 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     if constexpr (i % RS == 0 && i / RS < NR) {
                         issue_read(IntC<i / RS>{}, IntC<nx>{}, a_nx, b_nx);
                     }
-                    // DMA d of this k-step goes after MFMA d*NMFMA/dma_n (evenly spaced), one further on when the fragment
-                    // reads sit in the even gaps
+                    // DMA d of this k-step goes after MFMA d * DMA_STRIDE + 1 (hand-scheduled loops), else after MFMA
+                    // d*NMFMA/dma_n (evenly spaced; one further on when the fragment reads sit in the even gaps)
                     static_for<0, dma_n>([&](auto dc) {
-                        constexpr int slot = (dc.value * NMFMA) / dma_n + ((NMFMA / dma_n) >= 2 && RS % 2 == 0 ? 1 : 0);
+                        constexpr int slot = LATE ? dc.value * DMA_STRIDE + 1
+                                                  : (dc.value * NMFMA) / dma_n + ((NMFMA / dma_n) >= 2 && RS % 2 == 0 ? 1 : 0);
                         constexpr int j = Cfg::dma_index(dma_lo + dc.value);
                         if constexpr (ASM_DMA) {
                             constexpr bool is_a = j < A_DMA;

@@ -144,19 +144,20 @@ def _branch_free_loops(lines):
                 yield body
 
 
-def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled):
-    """The K loop of the largest tile issues its DMAs through inline assembly: `s_mov_b32 m0, <LDS base>` in one MFMA gap,
+@pytest.mark.parametrize("unit,dmas_per_k_tile", [("gemm_mfma_inst_256x256.hip", 16), ("gemm_mfma_inst_192x128.hip", 10)])
+def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled, unit, dmas_per_k_tile):
+    """The K loops of the larger tiles issue their DMAs through inline assembly: `s_mov_b32 m0, <LDS base>` in one MFMA gap,
     the `buffer_load_dwordx4 ... lds` that reads M0 in the next (`s_add_i32 m0, <base>, <constant>` for all but the first).  The compiler does not know M0 is live in between, so
     nothing else may write M0 there: in the steady loop of every whole-tile build each DMA must be preceded by exactly
     one write of M0 since the DMA before it, that write must be the hand-placed move, and an MFMA (the wait state the
     write needs) must lie between the two.  (The general iterations at either end of the K loop run the same source with
     the DMAs under run-time flags; their branches make a linear reading of the listing meaningless.)"""
-    asm, _ = compiled["gemm_mfma_inst_256x256.hip"]
+    asm, _ = compiled[unit]
     checked = 0
     for name, lines in _kernels(asm):
         if "Lb1ELb0ELi0EEEvNS_8GemmArgsE" in name:  # range-checked builds keep the compiler's own DMA
             continue
-        loops = [b for b in _branch_free_loops(lines) if sum(x.startswith("v_mfma") for x in b) >= 64]
+        loops = [b for b in _branch_free_loops(lines) if sum(x.startswith("v_mfma") for x in b) >= 48]
         assert loops, name[-40:]
         for body in loops:
             # (the loop is a cycle: start reading at its first DMA so that the write ahead of it is seen at the end)
@@ -176,6 +177,6 @@ def test_hand_placed_dma_finds_its_lds_base_in_m0(compiled):
                     assert len(writes) == 1 and re.match(r"s_(mov_b32 m0, s\d+|add_i32 m0, s\d+, 0x[0-9a-f]+)$", writes[0]), (name[-40:], writes)
                     assert mfma_since_write >= 1, name[-40:]
                     writes = []
-            assert dmas == 16, (name[-40:], dmas)
+            assert dmas == dmas_per_k_tile, (name[-40:], dmas)
             checked += 1
     assert checked >= 10
