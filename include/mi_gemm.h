@@ -185,6 +185,32 @@ int mi_matmul_f32_workspace_bytes(const mi_gemm_tensors* t, int precision, size_
 int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int tile, void* d_workspace,
                      size_t workspace_bytes, void* hip_stream);
 
+/* The C entry points that the reference's Exo procs compile to, with their argument lists:
+ *   xgemm_Sm80_fence / xgemm_Sm80_mbarrier (ctxt, M, N, K, A f32[M,K], B f32[K,N], C f32[M,N])      xgemm_Sm80.py:18-21
+ *   xgemm_Sm90_wgmma_n{64,128,256}[_tma_to_gmem|_split_k]
+ *       (ctxt, L, M, N, K_splits, cluster_k, A f32[L,M,K_splits,cluster_k], B f32[L,N,K_splits,cluster_k],
+ *        C f32[L,N,M])                                                                           xgemm_Sm90.py:43-48
+ * called at gemm/gemm_test.cu:288-294,326-362 (the Sm90 ones with the operands swapped, so that C[L,N,M] comes out as
+ * the harness's row-major M x N).  All tensors are dense and row-major in the order written; K = K_splits * cluster_k.
+ * The reference passes ctxt = nullptr, its generated code needing nothing from the caller.  This library never
+ * allocates, so here ctxt brings the scratch memory the fp32 operands are converted into, and the stream (the
+ * reference runs these on stream 0 only, gemm/gemm_test.cu:289,325).  K_splits > 1 selects what the reference's
+ * split-K build does - C zero-filled, K partitions added into it (xgemm_Sm90.py:60-61) - with the number of
+ * partitions chosen by the planner; the sum is the same.  The procs' divisibility assertions (M % 192, N % 256,
+ * K % 16, cluster_k % 4) are limits of those kernels, not of the interface: every positive size is accepted.
+ * L problems run in one launch after one conversion pass over each operand. */
+typedef struct mi_xgemm_context {
+    void* d_workspace;      /* 256-byte aligned device memory, at least mi_xgemm_workspace_bytes(...) */
+    size_t workspace_bytes;
+    void* hip_stream;
+    int precision;          /* MI_F32_BF16X1 | MI_F32_BF16X3 */
+    int tile;               /* MI_TILE_AUTO, or the tile that stands for an n64 / n128 / n256 variant */
+} mi_xgemm_context;
+int mi_xgemm_workspace_bytes(int L, int M, int N, int K, int precision, size_t* out_bytes);
+int mi_xgemm_Sm80(const mi_xgemm_context* ctxt, int M, int N, int K, const float* A, const float* B, float* C);
+int mi_xgemm_Sm90_wgmma(const mi_xgemm_context* ctxt, int L, int M, int N, int K_splits, int cluster_k, const float* A,
+                        const float* B, float* C);
+
 /* Diagnostic: the launch mi_matmul_mfma would make, with every workgroup recording time stamps so that a host tool
  * can show where a launch spends its time (per phase, per workgroup, per XCD).  Complements the whole-launch event
  * timing of the reference harness (gemm/gemm_test.cu:392-404), which has no in-kernel view.  Workgroup g writes
@@ -244,6 +270,11 @@ enum { MI_DATA_RANDOM = 0, MI_DATA_IDENTITY = 1, MI_DATA_TILED_NUMBERS = 2, MI_D
  * transpose_rule as in the reference (gemm_test.cu:64-65).  seed is used by styles 3 and 4 only. */
 int mi_init_test_data(void* d_tensor, uint32_t rows, uint32_t cols, int data_code, int transpose_rule,
                       int ab_dtype, double param, uint32_t seed, void* hip_stream);
+
+/* 16-bit elements widened to fp32, exactly: lets the fp32 entry points run on the values of a 16-bit test tensor, so
+ * that their results can be held against the same baseline (the reference's harness keeps every tensor in fp32,
+ * gemm/gemm_test.cu:218-226). */
+int mi_widen_to_f32(const void* d_src, int ab_dtype, float* d_dst, size_t count, void* hip_stream);
 
 /* Replaces `launch_device_compare_tensor` (gemm/gemm_test.cu:177-187): compares two rows x cols fp32 tensors
  * with the reference's rule (same sign, ratio < 1+1/32, gemm_test.cu:138-147) and additionally accumulates

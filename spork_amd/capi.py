@@ -79,6 +79,18 @@ def exported_symbols() -> list[str]:
     return sorted(set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)))
 
 
+class XgemmContext(C.Structure):
+    """Mirror of ``mi_xgemm_context``: what the `ctxt` argument of the xgemm entry points brings."""
+
+    _fields_ = [
+        ("d_workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
+        ("hip_stream", C.c_void_p),
+        ("precision", C.c_int),
+        ("tile", C.c_int),
+    ]
+
+
 _lib = None
 
 
@@ -118,6 +130,11 @@ def lib() -> C.CDLL:
     sig("mi_mfma_ceiling", i32, [vp, sz, i32, i32, u32, vp, vp, C.POINTER(u32), C.POINTER(C.c_double), vp])
     sig("mi_matmul_f32_workspace_bytes", i32, [tp, i32, C.POINTER(sz)])
     sig("mi_matmul_f32_ws", i32, [tp, i32, i32, i32, vp, sz, vp])
+    xp = C.POINTER(XgemmContext)
+    sig("mi_xgemm_workspace_bytes", i32, [i32, i32, i32, i32, i32, C.POINTER(sz)])
+    sig("mi_xgemm_Sm80", i32, [xp, i32, i32, i32, vp, vp, vp])
+    sig("mi_xgemm_Sm90_wgmma", i32, [xp, i32, i32, i32, i32, i32, vp, vp, vp])
+    sig("mi_widen_to_f32", i32, [vp, i32, vp, sz, vp])
     sig("mi_tile_name", C.c_char_p, [i32])
     sig("mi_tile_count", i32, [])
     sig("mi_tile_shape", i32, [i32, C.POINTER(u32), C.POINTER(u32), ip, ip])
@@ -240,6 +257,29 @@ def matmul_f32_ws(t: GpuTensors, workspace_ptr: int, workspace_bytes: int, preci
     """fp32 A and B (ab_dtype = F32), converted on the device to one or three bf16 terms in the caller's workspace."""
     check(lib().mi_matmul_f32_ws(C.byref(t), precision, k_mode, tile, workspace_ptr, workspace_bytes, stream),
           "mi_matmul_f32_ws")
+
+
+def xgemm_workspace_bytes(L: int, M: int, N: int, K: int, precision: int = F32_BF16X3) -> int:
+    n = C.c_size_t()
+    check(lib().mi_xgemm_workspace_bytes(L, M, N, K, precision, C.byref(n)), "mi_xgemm_workspace_bytes")
+    return n.value
+
+
+def xgemm_Sm80(ctxt: XgemmContext | None, M: int, N: int, K: int, a_ptr: int, b_ptr: int, c_ptr: int) -> None:
+    """Argument list of xgemm_Sm80_fence / _mbarrier (xgemm_Sm80.py:18-21): A f32[M,K], B f32[K,N], C f32[M,N]."""
+    check(lib().mi_xgemm_Sm80(C.byref(ctxt) if ctxt is not None else None, M, N, K, a_ptr, b_ptr, c_ptr), "mi_xgemm_Sm80")
+
+
+def xgemm_Sm90_wgmma(ctxt: XgemmContext | None, L: int, M: int, N: int, K_splits: int, cluster_k: int, a_ptr: int,
+                     b_ptr: int, c_ptr: int) -> None:
+    """Argument list of xgemm_Sm90_wgmma_* (xgemm_Sm90.py:43-48): A f32[L,M,K], B f32[L,N,K], C f32[L,N,M] with
+    K = K_splits * cluster_k."""
+    check(lib().mi_xgemm_Sm90_wgmma(C.byref(ctxt) if ctxt is not None else None, L, M, N, K_splits, cluster_k, a_ptr, b_ptr,
+                                    c_ptr), "mi_xgemm_Sm90_wgmma")
+
+
+def widen_to_f32(src_ptr: int, dtype: int, dst_ptr: int, count: int, stream: int = 0) -> None:
+    check(lib().mi_widen_to_f32(src_ptr, dtype, dst_ptr, count, stream), "mi_widen_to_f32")
 
 
 def matmul_mfma_timeline(t: GpuTensors, stamps_ptr: int, slots_per_workgroup: int, max_workgroups: int,

@@ -8,6 +8,7 @@
 //   gemm --versus llm|random    the planner against hipBLASLt over many shapes, with a summary table
 //   gemm --one M N K [f16|bf16] [data style 1..5] [param]    the planner (without and with workspace) and hipBLASLt on one shape
 //   gemm --kmodes M N K [f16|bf16] [style] [param]  one size: the planner, each K mode forced, hipBLASLt
+//   gemm --exo M N K [f16|bf16] [style] [param]     one size: the planner and every Exo-named fp32 entry point
 //   gemm --timeline M N K [f16|bf16] [tile code]    in-kernel timeline of one launch
 //   gemm --ceiling  what a register-only MFMA loop sustains on the benchmark's operand values
 #include <math.h>
@@ -26,7 +27,8 @@ int main(int argc, char** argv)
     const bool rounds = argc > 1 && strcmp(argv[1], "--rounds") == 0;
     const bool versus = argc > 2 && strcmp(argv[1], "--versus") == 0;
     const bool kmodes = argc > 1 && strcmp(argv[1], "--kmodes") == 0;  // --one with every K mode as a row of its own
-    const bool one = kmodes || (argc > 1 && strcmp(argv[1], "--one") == 0);
+    const bool exo = argc > 1 && strcmp(argv[1], "--exo") == 0;  // --one with the Exo-named entry points as rows
+    const bool one = kmodes || exo || (argc > 1 && strcmp(argv[1], "--one") == 0);
     int device_count = 0;
     if (mi_rt_device_count(&device_count) != MI_OK || device_count == 0) {
         fprintf(stderr, "no GPU visible\n");
@@ -73,7 +75,7 @@ int main(int argc, char** argv)
 
     // data_style 0: all three reference styles; 1: tiled x identity; 2: identity x tiled; 3: reference random;
     // 4: uniform[-param, param]; 5: normal(0,1)/sqrt(K)
-    auto sized_tests = [&failures, &keep_bits, &out_ms](uint32_t M, uint32_t N, uint32_t K, int data_style, int ab_dtype, double param = 1.0) {
+    auto sized_tests = [&failures, &keep_bits, &out_ms, exo_rows = exo](uint32_t M, uint32_t N, uint32_t K, int data_style, int ab_dtype, double param = 1.0) {
         TestParams params{};
         params.M = M;
         params.N = N;
@@ -111,6 +113,14 @@ int main(int argc, char** argv)
             }
         }
         params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_row_major_b);  // any shape, any layout
+        // fp32 operands are re-packed anyway: any shape; the n128 / n64 / K2 rows only where asked for (--exo)
+        params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::exo_sm_80_fence) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n256);
+        if (exo_rows) {
+            params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::exo_sm_90_n128) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n64);
+            if (K % 2 == 0) {
+                params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::exo_sm_90_n256_K2);
+            }
+        }
         if (hipblaslt_enabled()) {
             params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::hipblaslt);
         }
@@ -179,6 +189,11 @@ int main(int argc, char** argv)
         }
         keep_bits = algorithm_code_bit(AlgorithmCode::mi355_auto) | algorithm_code_bit(AlgorithmCode::mi355_auto_ws) |
                     algorithm_code_bit(AlgorithmCode::hipblaslt);
+        if (exo) {
+            keep_bits = algorithm_code_bit(AlgorithmCode::mi355_auto) | algorithm_code_bit(AlgorithmCode::exo_sm_80_fence) |
+                        algorithm_code_bit(AlgorithmCode::exo_sm_90_n256) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n256_K2) |
+                        algorithm_code_bit(AlgorithmCode::exo_sm_90_n128) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n64);
+        }
         if (kmodes) {
             keep_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum) |
                          algorithm_code_bit(AlgorithmCode::mi355_stream_k);

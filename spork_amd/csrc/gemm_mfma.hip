@@ -1233,9 +1233,10 @@ struct F32Prepared {
     size_t ws_b, ws_bytes;     // A copy at 0, B copy at ws_b
 };
 
-static int prepare_f32(const mi_gemm_tensors* t, int precision, F32Prepared& f)
+// `batches` problems of t's shape whose converted copies lie one after the other
+static int prepare_f32(const mi_gemm_tensors* t, int precision, F32Prepared& f, uint32_t batches = 1)
 {
-    if (!t || t->ab_dtype != MI_F32 || (precision != MI_F32_BF16X1 && precision != MI_F32_BF16X3)) {
+    if (!t || t->ab_dtype != MI_F32 || (precision != MI_F32_BF16X1 && precision != MI_F32_BF16X3) || batches == 0) {
         return MI_ERR_BAD_ARGUMENT;
     }
     mi_gemm_tensors probe = *t;
@@ -1252,8 +1253,8 @@ static int prepare_f32(const mi_gemm_tensors* t, int precision, F32Prepared& f)
     if (depth >= (1u << 21)) {
         return MI_ERR_UNSUPPORTED;
     }
-    f.ws_b = round_up((size_t)t->M * depth * 2, 256);
-    f.ws_bytes = f.ws_b + round_up((size_t)t->N * depth * 2, 256);
+    f.ws_b = round_up((size_t)batches * t->M * depth * 2, 256);
+    f.ws_bytes = f.ws_b + round_up((size_t)batches * t->N * depth * 2, 256);
     f.bf16 = *t;
     f.bf16.ab_dtype = MI_BF16;
     f.bf16.K = (uint32_t)depth;
@@ -1275,12 +1276,17 @@ int mi_matmul_f32_workspace_bytes(const mi_gemm_tensors* t, int precision, size_
     return MI_OK;
 }
 
-int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int tile, void* d_workspace, size_t workspace_bytes,
-                     void* hip_stream)
+// `batches` problems, densely packed (A[L,M,K], B[L,N,K] and C[L,..]); more than one only with both operands K-contiguous,
+// where the L matrices of an operand read as one matrix of L times the rows.
+static int run_f32(const mi_gemm_tensors* t, uint32_t batches, int precision, int k_mode, int tile, void* d_workspace,
+                   size_t workspace_bytes, void* hip_stream)
 {
     F32Prepared f;
-    if (const int st = prepare_f32(t, precision, f)) {
+    if (const int st = prepare_f32(t, precision, f, batches)) {
         return st;
+    }
+    if (batches > 1 && (t->a_col_major || !t->b_col_major)) {
+        return MI_ERR_UNSUPPORTED;
     }
     if (!d_workspace || workspace_bytes < f.ws_bytes || (uintptr_t)d_workspace % 256) {
         return MI_ERR_WORKSPACE;
@@ -1310,13 +1316,20 @@ int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int ti
     } ops[2] = {{t->a, const_cast<void*>(f.bf16.a), t->M, !t->a_col_major, a_lo_mask},
                 {t->b, const_cast<void*>(f.bf16.b), t->N, t->b_col_major != 0, b_lo_mask}};
     for (const auto& op : ops) {
-        const dim3 grid((f.kp + 63) / 64, (op.rows + 63) / 64, 1);
-        if (grid.y > 65535u) {
+        if (((uint64_t)batches * op.rows + 63) / 64 > 65535u) {
             return MI_ERR_UNSUPPORTED;
         }
-        hipLaunchKernelGGL(split_f32_kernel, grid, dim3(256), 0, stream, (const float*)op.src, (uint16_t*)op.dst, op.rows,
-                           t->K, f.kp, op.k_contiguous, f.terms, op.lo_mask);
+    }
+    for (const auto& op : ops) {
+        const uint32_t rows = batches * op.rows;
+        const dim3 grid((f.kp + 63) / 64, (rows + 63) / 64, 1);
+        hipLaunchKernelGGL(split_f32_kernel, grid, dim3(256), 0, stream, (const float*)op.src, (uint16_t*)op.dst, rows, t->K,
+                           f.kp, op.k_contiguous, f.terms, op.lo_mask);
         MI_CHECK_LAUNCH();
+    }
+    if (batches > 1) {
+        const BatchRequest req{batches, (uint64_t)t->M * f.bf16.K, (uint64_t)t->N * f.bf16.K, (uint64_t)t->M * t->N};
+        return run_mfma(&f.bf16, k_mode, tile, nullptr, 0, hip_stream, nullptr, &req);
     }
     // what the converted operands leave of the workspace may hold K partitions' copies of C
     const size_t used = round_up(f.ws_bytes, 256);
@@ -1324,6 +1337,81 @@ int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int ti
         return run_mfma(&f.bf16, k_mode, tile, (char*)d_workspace + used, workspace_bytes - used, hip_stream);
     }
     return run_mfma(&f.bf16, k_mode, tile, nullptr, 0, hip_stream);
+}
+
+int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int tile, void* d_workspace, size_t workspace_bytes,
+                     void* hip_stream)
+{
+    return run_f32(t, 1, precision, k_mode, tile, d_workspace, workspace_bytes, hip_stream);
+}
+
+// The operand bundle of one xgemm problem, or an error for sizes the reference's procs assert away
+// (xgemm_Sm80.py:19-21, xgemm_Sm90.py:49-54: every size positive).
+static int xgemm_tensors(int64_t M, int64_t N, int64_t K, const float* a, const float* b, float* c, bool b_col_major,
+                         bool c_col_major, mi_gemm_tensors& t)
+{
+    if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    t = mi_gemm_tensors{};
+    t.M = (uint32_t)M;
+    t.N = (uint32_t)N;
+    t.K = (uint32_t)K;
+    t.a = a;
+    t.b = b;
+    t.c = c;
+    t.a_col_major = 0;
+    t.b_col_major = b_col_major;
+    t.c_col_major = c_col_major;
+    t.ab_dtype = MI_F32;
+    return MI_OK;
+}
+
+int mi_xgemm_workspace_bytes(int L, int M, int N, int K, int precision, size_t* out_bytes)
+{
+    mi_gemm_tensors t;
+    F32Prepared f;
+    if (!out_bytes || L <= 0) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    // (sizes only: the pointers are placeholders that pass the alignment checks)
+    alignas(256) static const float placeholder[64] = {};
+    if (const int st = xgemm_tensors(M, N, K, placeholder, placeholder, const_cast<float*>(placeholder), true, true, t)) {
+        return st;
+    }
+    if (const int st = prepare_f32(&t, precision, f, (uint32_t)L)) {
+        return st;
+    }
+    *out_bytes = f.ws_bytes;
+    return MI_OK;
+}
+
+int mi_xgemm_Sm80(const mi_xgemm_context* ctxt, int M, int N, int K, const float* A, const float* B, float* C)
+{
+    mi_gemm_tensors t;
+    if (!ctxt) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    if (const int st = xgemm_tensors(M, N, K, A, B, C, false, false, t)) {
+        return st;
+    }
+    return run_f32(&t, 1, ctxt->precision, MI_K_AUTO, ctxt->tile, ctxt->d_workspace, ctxt->workspace_bytes, ctxt->hip_stream);
+}
+
+int mi_xgemm_Sm90_wgmma(const mi_xgemm_context* ctxt, int L, int M, int N, int K_splits, int cluster_k, const float* A,
+                        const float* B, float* C)
+{
+    mi_gemm_tensors t;
+    if (!ctxt || L <= 0 || K_splits <= 0 || cluster_k <= 0) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    if (const int st = xgemm_tensors(M, N, (int64_t)K_splits * cluster_k, A, B, C, true, true, t)) {
+        return st;
+    }
+    // K_splits > 1 is the reference's split-K build, which zero-fills C and lets the K tasks add into it
+    // (xgemm_Sm90.py:60-61,65): the same request here, with the number of partitions left to the planner
+    return run_f32(&t, (uint32_t)L, ctxt->precision, K_splits > 1 ? MI_K_SPLIT : MI_K_AUTO, ctxt->tile, ctxt->d_workspace,
+                   ctxt->workspace_bytes, ctxt->hip_stream);
 }
 
 int mi_matmul_mfma_workspace_bytes(const mi_gemm_tensors* t, size_t* out_bytes)

@@ -80,6 +80,21 @@ int gemm_test(TestParams params, gpu_stream_t stream)
         matmul_baseline(t, stream);
     }
 
+    // The Exo entry points take fp32 tensors (gemm/gemm_test.cu:218-226 keeps everything in fp32): the same values,
+    // widened, so that their results are held against the same baseline.
+    const uint64_t exo_bits = algorithm_code_bit(AlgorithmCode::exo_sm_80_fence) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n256) |
+                              algorithm_code_bit(AlgorithmCode::exo_sm_90_n256_K2) | algorithm_code_bit(AlgorithmCode::exo_sm_90_n128) |
+                              algorithm_code_bit(AlgorithmCode::exo_sm_90_n64);
+    float *d_a32 = nullptr, *d_b32 = nullptr, *d_bCol32 = nullptr;
+    if (params.algorithm_code_bits & exo_bits) {
+        d_a32 = static_cast<float*>(device_alloc(4 * M * K));
+        d_b32 = static_cast<float*>(device_alloc(4 * N * K));
+        d_bCol32 = static_cast<float*>(device_alloc(4 * N * K));
+        gpu_check(mi_widen_to_f32(d_a, params.ab_dtype, d_a32, M * K, stream), "widen a");
+        gpu_check(mi_widen_to_f32(d_b, params.ab_dtype, d_b32, N * K, stream), "widen b");
+        gpu_check(mi_widen_to_f32(d_bCol, params.ab_dtype, d_bCol32, N * K, stream), "widen bCol");
+    }
+
     int failures = 0;
 
     // Test loop
@@ -128,6 +143,33 @@ int gemm_test(TestParams params, gpu_stream_t stream)
               case AlgorithmCode::mi355_stream_k:
                 matmul_mi355_any_layout(t, stream_ws, MI_K_STREAM, MI_TILE_AUTO);
                 break;
+              // gemm/gemm_test.cu:326,335,358,362 and :288-294: the Sm90 ones with the operands swapped, so that their
+              // C[L,N,M] is the row-major M x N of the harness
+              case AlgorithmCode::exo_sm_80_fence: {
+                mi_xgemm_context ctxt = xgemm_context(stream_ws, 1, int(params.M), int(params.N), int(params.K));
+                xgemm_Sm80_fence(&ctxt, int(params.M), int(params.N), int(params.K), d_a32, d_b32, d_c_tested);
+                break;
+              }
+              case AlgorithmCode::exo_sm_90_n256: {
+                mi_xgemm_context ctxt = xgemm_context(stream_ws, 1, int(params.N), int(params.M), int(params.K));
+                xgemm_Sm90_wgmma_n256(&ctxt, 1, int(params.N), int(params.M), 1, int(params.K), d_bCol32, d_a32, d_c_tested);
+                break;
+              }
+              case AlgorithmCode::exo_sm_90_n256_K2: {
+                mi_xgemm_context ctxt = xgemm_context(stream_ws, 1, int(params.N), int(params.M), int(params.K));
+                xgemm_Sm90_wgmma_n256_split_k(&ctxt, 1, int(params.N), int(params.M), 2, int(params.K / 2), d_bCol32, d_a32, d_c_tested);
+                break;
+              }
+              case AlgorithmCode::exo_sm_90_n128: {
+                mi_xgemm_context ctxt = xgemm_context(stream_ws, 1, int(params.N), int(params.M), int(params.K));
+                xgemm_Sm90_wgmma_n128(&ctxt, 1, int(params.N), int(params.M), 1, int(params.K), d_bCol32, d_a32, d_c_tested);
+                break;
+              }
+              case AlgorithmCode::exo_sm_90_n64: {
+                mi_xgemm_context ctxt = xgemm_context(stream_ws, 1, int(params.N), int(params.M), int(params.K));
+                xgemm_Sm90_wgmma_n64(&ctxt, 1, int(params.N), int(params.M), 1, int(params.K), d_bCol32, d_a32, d_c_tested);
+                break;
+              }
               case AlgorithmCode::mi355_row_major_b: {
                 GPU_Tensors t_row{params.M, params.N, params.K, d_a, d_b, d_c_tested, 0, 0, 0, params.ab_dtype};
                 matmul_mi355_any_layout(t_row, stream_ws);
@@ -206,6 +248,11 @@ int gemm_test(TestParams params, gpu_stream_t stream)
     mi_rt_free(d_a);
     mi_rt_free(d_b);
     mi_rt_free(d_bCol);
+    if (d_a32) {
+        mi_rt_free(d_a32);
+        mi_rt_free(d_b32);
+        mi_rt_free(d_bCol32);
+    }
     mi_rt_free(d_c_baseline);
     mi_rt_free(d_c_tested);
     mi_rt_free(d_result);

@@ -29,6 +29,11 @@ enum class AlgorithmCode
     mi355_split_k_sum,    // K split forced, partitions summed from copies of C in the workspace (no atomics)
     mi355_stream_k,       // stream-K forced: equal runs of (tile, K tile) pairs, parts summed from the workspace
     hipblaslt,            // vendor comparator (the cuBLAS / CUTLASS rows of gemm/gemm_test.h:19-20)
+    exo_sm_80_fence,      // the reference's Exo entry points by name (gemm/gemm_test.h:21-31), on the test data widened
+    exo_sm_90_n256,       //   to fp32: three bf16 terms per product, so about 3.3x the 16-bit time
+    exo_sm_90_n256_K2,
+    exo_sm_90_n128,
+    exo_sm_90_n64,
     first_forced_tile,    // + (tile code - 1)
 };
 
@@ -78,6 +83,16 @@ inline const char* algorithm_name(AlgorithmCode code)
         return "mi355 (stream k)";
       case AlgorithmCode::hipblaslt:
         return "hipBLASLt";
+      case AlgorithmCode::exo_sm_80_fence:
+        return "exo_sm_80_fence (fp32 in, bf16x3)";
+      case AlgorithmCode::exo_sm_90_n256:
+        return "exo_sm_90_n256 (fp32 in, bf16x3)";
+      case AlgorithmCode::exo_sm_90_n256_K2:
+        return "exo_sm_90_n256_K2 (fp32 in, bf16x3)";
+      case AlgorithmCode::exo_sm_90_n128:
+        return "exo_sm_90_n128 (fp32 in, bf16x3)";
+      case AlgorithmCode::exo_sm_90_n64:
+        return "exo_sm_90_n64 (fp32 in, bf16x3)";
       default:
         break;
     }

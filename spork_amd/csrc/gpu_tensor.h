@@ -146,6 +146,57 @@ inline void matmul_mi355_any_layout(GPU_Tensors t, StreamWorkspace& stream_ws, i
     gpu_check(mi_matmul_mfma_ws(&abi, k_mode, tile, d_ws, preferred, stream_ws.stream), "matmul_mi355_any_layout");
 }
 
+// The entry points that the reference's Exo procs compile to, by their names and argument lists (proc signatures
+// xgemm_Sm80.py:18-21 and xgemm_Sm90.py:43-48, instances xgemm_Sm90_n{64,128,256}.py:3 and
+// xgemm_Sm90_n256_tma_to_gmem.py:3-4; called at gemm/gemm_test.cu:288-294,326-362).  The reference passes ctxt = nullptr;
+// here ctxt points to a mi_xgemm_context, which names the stream and the scratch memory that the fp32 operands are
+// converted into (xgemm_context below fills one from a StreamWorkspace).  The n64 / n128 / n256 instances differ in
+// their tile; here each stands for the tile of this chip's family nearest to it, unless ctxt->tile names one.  The
+// fence and mbarrier builds of the Sm80 proc, and the plain and tma_to_gmem builds of the Sm90 one, differ in how the
+// kernel synchronises and stores, not in what is computed: they are one call each here.
+inline mi_xgemm_context xgemm_context(StreamWorkspace& stream_ws, int L, int M, int N, int K, int precision = MI_F32_BF16X3,
+                                      int tile = MI_TILE_AUTO)
+{
+    size_t bytes = 0;
+    gpu_check(mi_xgemm_workspace_bytes(L, M, N, K, precision, &bytes), "xgemm_context (workspace size)");
+    return mi_xgemm_context{stream_ws.alloc_at_least(bytes), bytes, stream_ws.stream, precision, tile};
+}
+
+inline void xgemm_Sm80_fence(void* ctxt, int M, int N, int K, const float* A, const float* B, float* C)
+{
+    gpu_check(mi_xgemm_Sm80(static_cast<const mi_xgemm_context*>(ctxt), M, N, K, A, B, C), "xgemm_Sm80_fence");
+}
+
+inline void xgemm_Sm80_mbarrier(void* ctxt, int M, int N, int K, const float* A, const float* B, float* C)
+{
+    gpu_check(mi_xgemm_Sm80(static_cast<const mi_xgemm_context*>(ctxt), M, N, K, A, B, C), "xgemm_Sm80_mbarrier");
+}
+
+inline void xgemm_Sm90_wgmma_variant(const char* what, int namesake_tile, void* ctxt, int L, int M, int N, int K_splits,
+                                     int cluster_k, const float* A, const float* B, float* C)
+{
+    if (!ctxt) {
+        gpu_check(MI_ERR_BAD_ARGUMENT, what);
+    }
+    mi_xgemm_context with_tile = *static_cast<const mi_xgemm_context*>(ctxt);
+    if (with_tile.tile == MI_TILE_AUTO) {
+        with_tile.tile = namesake_tile;
+    }
+    gpu_check(mi_xgemm_Sm90_wgmma(&with_tile, L, M, N, K_splits, cluster_k, A, B, C), what);
+}
+
+#define MI_XGEMM_SM90_INSTANCE(name, namesake_tile)                                                                          \
+    inline void name(void* ctxt, int L, int M, int N, int K_splits, int cluster_k, const float* A, const float* B, float* C) \
+    {                                                                                                                        \
+        xgemm_Sm90_wgmma_variant(#name, namesake_tile, ctxt, L, M, N, K_splits, cluster_k, A, B, C);                         \
+    }
+MI_XGEMM_SM90_INSTANCE(xgemm_Sm90_wgmma_n256, MI_TILE_256x256)
+MI_XGEMM_SM90_INSTANCE(xgemm_Sm90_wgmma_n256_tma_to_gmem, MI_TILE_256x256)
+MI_XGEMM_SM90_INSTANCE(xgemm_Sm90_wgmma_n256_split_k, MI_TILE_256x256)
+MI_XGEMM_SM90_INSTANCE(xgemm_Sm90_wgmma_n128, MI_TILE_256x128)
+MI_XGEMM_SM90_INSTANCE(xgemm_Sm90_wgmma_n64, MI_TILE_64x128)
+#undef MI_XGEMM_SM90_INSTANCE
+
 // Vendor comparator, shaped like matmul_cutlass / cutlass_enabled (gemm/cutlass_gemm.h:5-6).
 inline bool hipblaslt_enabled()
 {

@@ -91,6 +91,13 @@ __global__ __launch_bounds__(256) void init_test_data_kernel(uint16_t* d_tensor,
     }
 }
 
+__global__ __launch_bounds__(256) void widen_kernel(const uint16_t* d_src, int dtype, float* d_dst, size_t count)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+        d_dst[i] = widen16(d_src[i], dtype);
+    }
+}
+
 __global__ void compare_init_kernel(unsigned long long* d_result)
 {
     d_result[0] = ~0ull;
@@ -158,6 +165,19 @@ int mi_init_test_data(void* d_tensor, uint32_t rows, uint32_t cols, int data_cod
     gy = gy > 4096u ? 4096u : gy;
     hipLaunchKernelGGL(init_test_data_kernel, dim3(gx, gy, 1), dim3(256, 1, 1), 0, as_stream(hip_stream),
                        (uint16_t*)d_tensor, rows, cols, data_code, transpose_rule, ab_dtype, param, seed);
+    MI_CHECK_LAUNCH();
+    return MI_OK;
+}
+
+int mi_widen_to_f32(const void* d_src, int ab_dtype, float* d_dst, size_t count, void* hip_stream)
+{
+    if (!d_src || !d_dst || count == 0 || (ab_dtype != MI_F16 && ab_dtype != MI_BF16)) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    size_t blocks = (count + 255) / 256;
+    blocks = blocks > 8192 ? 8192 : blocks;
+    hipLaunchKernelGGL(widen_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(hip_stream), (const uint16_t*)d_src,
+                       ab_dtype, d_dst, count);
     MI_CHECK_LAUNCH();
     return MI_OK;
 }

@@ -339,6 +339,43 @@ def test_f32_entry_sizes_and_validation():
     assert lib.mi_matmul_f32_ws(C.byref(t), S.F32_BF16X3, 9, S.TILE_AUTO, 4096, need, None) == 2
 
 
+def test_xgemm_entries_sizes_and_validation():
+    """The entry points with the argument lists of the reference's Exo-generated C (xgemm_Sm80.py:18-21,
+    xgemm_Sm90.py:43-54): what they refuse before any device call."""
+    lib = S.lib()
+    up = lambda x: (x + 255) // 256 * 256
+    # the shape of the reference's own sync check (xgemm_Sm90.py:203): L = 2, M = 500, N = 800, K = 2 * 240
+    assert S.xgemm_workspace_bytes(2, 500, 800, 480) == up(2 * 500 * 1440 * 2) + up(2 * 800 * 1440 * 2)
+    assert S.xgemm_workspace_bytes(1, 500, 800, 480, S.F32_BF16X1) == up(500 * 480 * 2) + up(800 * 480 * 2)
+    n = C.c_size_t()
+    for bad in ((0, 8, 8, 8), (1, 0, 8, 8), (1, 8, -1, 8), (1, 8, 8, 0)):
+        assert lib.mi_xgemm_workspace_bytes(*bad, S.F32_BF16X3, C.byref(n)) == 2, bad
+    assert lib.mi_xgemm_workspace_bytes(1, 8, 8, 8, S.F32_BF16X3, None) == 2
+    assert lib.mi_xgemm_workspace_bytes(1, 8, 8, 8, 5, C.byref(n)) == 2
+    assert C.sizeof(S.XgemmContext) == 32 and S.XgemmContext.precision.offset == 24 and S.XgemmContext.tile.offset == 28
+    need = S.xgemm_workspace_bytes(1, 192, 256, 64)
+    ctxt = S.XgemmContext(4096, need, None, S.F32_BF16X3, S.TILE_AUTO)
+    p = 4096  # placeholder addresses: every call below is refused before anything is launched
+    assert lib.mi_xgemm_Sm80(None, 192, 256, 64, p, p, p) == 2                        # the context is not optional
+    assert lib.mi_xgemm_Sm80(C.byref(ctxt), 0, 256, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm80(C.byref(ctxt), 192, 256, 64, None, p, p) == 2
+    assert lib.mi_xgemm_Sm90_wgmma(None, 1, 192, 256, 1, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 0, 192, 256, 1, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 1, 192, 256, 0, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 1, 192, 256, 1, 0, p, p, p) == 2
+    small = S.XgemmContext(4096, need - 1, None, S.F32_BF16X3, S.TILE_AUTO)
+    assert lib.mi_xgemm_Sm80(C.byref(small), 192, 256, 64, p, p, p) == 3
+    assert lib.mi_xgemm_Sm90_wgmma(C.byref(small), 1, 192, 256, 1, 64, p, p, p) == 3
+    assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 2, 192, 256, 1, 64, p, p, p) == 3   # two problems need twice the room
+    unaligned = S.XgemmContext(4096 + 64, need, None, S.F32_BF16X3, S.TILE_AUTO)
+    assert lib.mi_xgemm_Sm80(C.byref(unaligned), 192, 256, 64, p, p, p) == 3
+    bad_tile = S.XgemmContext(4096, need, None, S.F32_BF16X3, 99)
+    assert lib.mi_xgemm_Sm80(C.byref(bad_tile), 192, 256, 64, p, p, p) == 2
+    assert lib.mi_widen_to_f32(None, S.BF16, p, 16, None) == 2
+    assert lib.mi_widen_to_f32(p, S.F32, p, 16, None) == 2
+    assert lib.mi_widen_to_f32(p, S.F16, p, 0, None) == 2
+
+
 def test_ceiling_probe_validates_its_arguments():
     lib = S.lib()
     n, f = C.c_uint32(), C.c_double()

@@ -543,6 +543,85 @@ def test_f32_inputs_known_answer(gpu):
         assert torch.equal(c, want)
 
 
+def _xgemm_ctxt(gpu, L, M, N, K, precision, tile=0, slack=0):
+    need = gpu.xgemm_workspace_bytes(L, M, N, K, precision)
+    ws = torch.empty(need + slack, dtype=torch.uint8, device="cuda")
+    return gpu.XgemmContext(ws.data_ptr(), need + slack, H.stream_handle(), precision, tile), ws
+
+
+@pytest.mark.parametrize("precision,tol", [("F32_BF16X3", 3e-5), ("F32_BF16X1", 1e-2)])
+@pytest.mark.parametrize("shape", [(192, 256, 64), (384, 512, 1024), (300, 200, 100)])
+def test_xgemm_sm80_argument_list(gpu, precision, tol, shape):
+    """xgemm_Sm80_fence(ctxt, M, N, K, A f32[M,K], B f32[K,N], C f32[M,N]) (xgemm_Sm80.py:18-21, called at
+    gemm/gemm_test.cu:326): against numpy's float64 product, on the proc's smallest legal shape (one 192 x 256 tile,
+    K % 16), a multiple of it, and a shape its assertions exclude but the interface admits."""
+    import numpy as np
+
+    M, N, K = shape
+    g = torch.Generator(device="cuda").manual_seed(80)
+    a = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32)
+    b = torch.randn((K, N), generator=g, device="cuda", dtype=torch.float32)
+    c = H.poisoned_c(M, N)
+    ctxt, _ws = _xgemm_ctxt(gpu, 1, M, N, K, getattr(gpu, precision))
+    gpu.xgemm_Sm80(ctxt, M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    ref = a.cpu().numpy().astype(np.float64) @ b.cpu().numpy().astype(np.float64)
+    assert H.rel_err(c.cpu().numpy(), ref) < tol
+
+
+@pytest.mark.parametrize("case", [
+    # L, M, N, K_splits, cluster_k, tile
+    (2, 500, 800, 1, 240, "TILE_AUTO"),      # the reference's own check of the proc (xgemm_Sm90.py:203)
+    (2, 500, 800, 2, 240, "TILE_AUTO"),      # ... and of its split-K build (:202)
+    (1, 512, 384, 1, 1024, "TILE_256x256"),  # L = 1, as the harness calls it (gemm/gemm_test.cu:335)
+    (1, 256, 256, 8, 512, "TILE_128x128"),   # the harness's K splits (gemm/gemm_test.cu:341-355)
+    (5, 64, 72, 1, 36, "TILE_AUTO"),         # many small ragged problems in one launch
+    (3, 200, 136, 4, 68, "TILE_64x128"),     # split K zero-fills every problem's C
+])
+def test_xgemm_sm90_argument_list(gpu, case):
+    """xgemm_Sm90_wgmma(ctxt, L, M, N, K_splits, cluster_k, A f32[L,M,K], B f32[L,N,K], C f32[L,N,M])
+    (xgemm_Sm90.py:43-48): every problem against numpy's float64 product of its own slices; C arrives poisoned, so the
+    split-K cases also show that the entry zero-fills before the partitions add (xgemm_Sm90.py:60-61)."""
+    import numpy as np
+
+    L, M, N, K_splits, cluster_k, tile = case
+    K = K_splits * cluster_k
+    g = torch.Generator(device="cuda").manual_seed(90)
+    a = torch.randn((L, M, K), generator=g, device="cuda", dtype=torch.float32)
+    b = torch.randn((L, N, K), generator=g, device="cuda", dtype=torch.float32)
+    c = torch.empty((L, N, M), dtype=torch.float32, device="cuda")
+    c.view(torch.uint8).fill_(0x7D)
+    ctxt, _ws = _xgemm_ctxt(gpu, L, M, N, K, gpu.F32_BF16X3, getattr(gpu, tile))
+    gpu.xgemm_Sm90_wgmma(ctxt, L, M, N, K_splits, cluster_k, a.data_ptr(), b.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    ha, hb, hc = a.cpu().numpy().astype(np.float64), b.cpu().numpy().astype(np.float64), c.cpu().numpy()
+    for l in range(L):
+        assert H.rel_err(hc[l], hb[l] @ ha[l].T) < 3e-5, l
+
+
+def test_xgemm_sm90_as_the_harness_calls_it(gpu, oracle):
+    """The reference's harness passes (1, N, M, 1, K, B column-major, A, C) - operands swapped - so that C[L,N,M] is its
+    row-major M x N (gemm/gemm_test.cu:335).  The same call here on 16-bit test data widened to fp32 gives what the
+    16-bit entry point gives on the data itself, to fp32 rounding: bf16 values split into (value, 0) exactly."""
+    M, N, K = 320, 448, 512
+    dtype = gpu.BF16
+    a16 = H.gen_on_device(M, K, 3, False, dtype, 1.0, 1)
+    b16 = H.gen_on_device(N, K, 3, True, dtype, 1.0, 2)
+    a32 = torch.empty((M, K), dtype=torch.float32, device="cuda")
+    b32 = torch.empty((N, K), dtype=torch.float32, device="cuda")
+    st = H.stream_handle()
+    gpu.widen_to_f32(a16.data_ptr(), dtype, a32.data_ptr(), M * K, st)
+    gpu.widen_to_f32(b16.data_ptr(), dtype, b32.data_ptr(), N * K, st)
+    torch.cuda.synchronize()
+    assert torch.equal(a32, a16.view(torch.bfloat16).to(torch.float32).reshape(M, K))
+    c = H.poisoned_c(M, N)
+    ctxt, _ws = _xgemm_ctxt(gpu, 1, N, M, K, gpu.F32_BF16X3)
+    gpu.xgemm_Sm90_wgmma(ctxt, 1, N, M, 1, K, b32.data_ptr(), a32.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    ref = oracle.gemm_f64(M, N, K, a16.cpu().numpy().view("uint16").reshape(M, K), b16.cpu().numpy().view("uint16").reshape(N, K), dtype)
+    assert H.rel_err(c.cpu().numpy(), ref) < 1e-5
+
+
 @pytest.mark.parametrize("tile", [16, 32])
 def test_mfma_ceiling_probe(gpu, tile):
     """The MFMA-only measurement loop runs on every CU, reports plausible clocks and the flop it performed; on zeros
