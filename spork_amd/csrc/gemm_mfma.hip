@@ -854,7 +854,8 @@ static int repack(const Operand& op, uint32_t K, void* dst, hipStream_t stream)
 
 // fp32 -> bf16 terms, K-contiguous rows of pitch terms*kp: segment s of a row holds the hi part (bf16 nearest to x)
 // or the lo part (bf16 nearest to x - hi) of the row's K values, zero-padded to kp.  `lo_mask` bit s selects lo.
-// Same 64 x 64 tiling as repack_kernel; a transposing read goes through LDS.
+// Three kernels: K-contiguous rows of any K and alignment (this one, element by element), K-contiguous rows with
+// K % 8 == 0 and 16-byte alignment, and operands stored K x rows.
 __device__ __forceinline__ uint16_t bf16_rne(float x)
 {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
@@ -866,28 +867,90 @@ __device__ __forceinline__ uint16_t bf16_rne(float x)
 }
 
 __global__ __launch_bounds__(256) void split_f32_kernel(const float* in, uint16_t* out, uint32_t rows, uint32_t K, uint32_t kp,
-                                                        int k_contiguous, uint32_t terms, uint32_t lo_mask)
+                                                        uint32_t terms, uint32_t lo_mask)
 {
-    __shared__ float tile[64][65];
     const uint32_t r0 = blockIdx.y * 64, k0 = blockIdx.x * 64;
     const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;
-    if (!k_contiguous) {
-        for (uint32_t kk = ty; kk < 64; kk += 4) {
-            const uint32_t k = k0 + kk, r = r0 + tx;
-            tile[kk][tx] = (k < K && r < rows) ? in[(size_t)k * rows + r] : 0.0f;
-        }
-        __syncthreads();
-    }
     for (uint32_t rr = ty; rr < 64; rr += 4) {
         const uint32_t r = r0 + rr, k = k0 + tx;
         if (r < rows && k < kp) {
-            const float x = k_contiguous ? (k < K ? in[(size_t)r * K + k] : 0.0f) : tile[tx][rr];
+            const float x = k < K ? in[(size_t)r * K + k] : 0.0f;
             const uint16_t hi = bf16_rne(x);
             const uint16_t lo = bf16_rne(x - __builtin_bit_cast(float, (uint32_t)hi << 16));
             uint16_t* const row = out + (size_t)r * terms * kp + k;
             for (uint32_t s = 0; s < terms; ++s) {
                 row[(size_t)s * kp] = (lo_mask >> s & 1u) ? lo : hi;
             }
+        }
+    }
+}
+
+// The same split for K-contiguous fp32 rows with K % 8 == 0 and 16-byte aligned rows: a lane takes eight consecutive values
+// of a row (two 16-byte loads) and writes one 16-byte store per term, so a wave reads 2 KB and writes 1 KB per term in
+// one piece.  `chunks` = rows * K / 8; the row pitch of `out` is terms * K.
+__global__ __launch_bounds__(256) void split_f32_rows_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
+                                                             uint64_t chunks, uint32_t chunks_per_row, uint32_t terms,
+                                                             uint32_t lo_mask)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    for (uint64_t c = (uint64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (uint64_t)gridDim.x * 256) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(in) + c * 2;
+        const f32x4 x0 = __builtin_nontemporal_load(src), x1 = __builtin_nontemporal_load(src + 1);
+        const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        uint32_t hi[4], lo[4];
+        for (int i = 0; i < 4; ++i) {
+            const uint16_t h0 = bf16_rne(x[2 * i]), h1 = bf16_rne(x[2 * i + 1]);
+            const uint16_t l0 = bf16_rne(x[2 * i] - __builtin_bit_cast(float, (uint32_t)h0 << 16));
+            const uint16_t l1 = bf16_rne(x[2 * i + 1] - __builtin_bit_cast(float, (uint32_t)h1 << 16));
+            hi[i] = (uint32_t)h0 | (uint32_t)h1 << 16;
+            lo[i] = (uint32_t)l0 | (uint32_t)l1 << 16;
+        }
+        const uint64_t row = c / chunks_per_row;
+        const uint32_t in_row = (uint32_t)(c - row * chunks_per_row);
+        u32x4* dst = reinterpret_cast<u32x4*>(out) + (row * terms) * chunks_per_row + in_row;
+        for (uint32_t s = 0; s < terms; ++s) {
+            dst[(uint64_t)s * chunks_per_row] = (lo_mask >> s & 1u) ? u32x4{lo[0], lo[1], lo[2], lo[3]} : u32x4{hi[0], hi[1], hi[2], hi[3]};
+        }
+    }
+}
+
+// The same split for fp32 operands stored K x rows (rows contiguous): 128 x 64 blocks are turned through LDS, so that
+// the reads are 256-byte row segments of the source and every lane writes eight consecutive K values (16 bytes) per
+// term.  Values beyond K (up to kp, the pitch of one term) are zeros.
+__global__ __launch_bounds__(256) void split_f32_transposed_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
+                                                                   uint32_t rows, uint32_t K, uint32_t kp, uint32_t terms,
+                                                                   uint32_t lo_mask)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ float tile[128][65];
+    // consecutive workgroups take neighbouring segments of the same 128 source rows
+    const uint32_t r0 = blockIdx.x * 64, k0 = blockIdx.y * 128;
+    const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    for (uint32_t kk = ty; kk < 128; kk += 4) {
+        const uint32_t k = k0 + kk, r = r0 + tx;
+        tile[kk][tx] = (k < K && r < rows) ? __builtin_nontemporal_load(in + (size_t)k * rows + r) : 0.0f;
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < 64 * 16; i += 256) {
+        const uint32_t rr = i / 16, ch = i % 16;
+        const uint32_t r = r0 + rr, k = k0 + ch * 8;
+        if (r >= rows || k >= kp) {
+            continue;
+        }
+        uint32_t hi[4], lo[4];
+        for (int j = 0; j < 4; ++j) {
+            const float x0 = tile[ch * 8 + 2 * j][rr], x1 = tile[ch * 8 + 2 * j + 1][rr];
+            const uint16_t h0 = bf16_rne(x0), h1 = bf16_rne(x1);
+            const uint16_t l0 = bf16_rne(x0 - __builtin_bit_cast(float, (uint32_t)h0 << 16));
+            const uint16_t l1 = bf16_rne(x1 - __builtin_bit_cast(float, (uint32_t)h1 << 16));
+            hi[j] = (uint32_t)h0 | (uint32_t)h1 << 16;
+            lo[j] = (uint32_t)l0 | (uint32_t)l1 << 16;
+        }
+        uint16_t* const row = out + (size_t)r * terms * kp + k;
+        for (uint32_t s = 0; s < terms; ++s) {
+            *reinterpret_cast<u32x4*>(row + (size_t)s * kp) =
+                (lo_mask >> s & 1u) ? u32x4{lo[0], lo[1], lo[2], lo[3]} : u32x4{hi[0], hi[1], hi[2], hi[3]};
         }
     }
 }
@@ -1322,9 +1385,23 @@ static int run_f32(const mi_gemm_tensors* t, uint32_t batches, int precision, in
     }
     for (const auto& op : ops) {
         const uint32_t rows = batches * op.rows;
+        if (op.k_contiguous && t->K % 8 == 0 && (uintptr_t)op.src % 16 == 0) {
+            const uint64_t chunks = (uint64_t)rows * (t->K / 8);
+            const uint64_t blocks = (chunks + 255) / 256;
+            hipLaunchKernelGGL(split_f32_rows_kernel, dim3((uint32_t)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream,
+                               (const float*)op.src, (uint16_t*)op.dst, chunks, t->K / 8, f.terms, op.lo_mask);
+            MI_CHECK_LAUNCH();
+            continue;
+        }
+        if (!op.k_contiguous) {
+            hipLaunchKernelGGL(split_f32_transposed_kernel, dim3((rows + 63) / 64, (f.kp + 127) / 128, 1), dim3(256), 0, stream,
+                               (const float*)op.src, (uint16_t*)op.dst, rows, t->K, f.kp, f.terms, op.lo_mask);
+            MI_CHECK_LAUNCH();
+            continue;
+        }
         const dim3 grid((f.kp + 63) / 64, (rows + 63) / 64, 1);
         hipLaunchKernelGGL(split_f32_kernel, grid, dim3(256), 0, stream, (const float*)op.src, (uint16_t*)op.dst, rows, t->K,
-                           f.kp, op.k_contiguous, f.terms, op.lo_mask);
+                           f.kp, f.terms, op.lo_mask);
         MI_CHECK_LAUNCH();
     }
     if (batches > 1) {

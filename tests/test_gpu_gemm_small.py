@@ -520,6 +520,28 @@ def test_f32_inputs(gpu, precision, tol, layout, shape):
         gpu.matmul_f32_ws(t, ws.data_ptr(), need - 1, prec, gpu.K_AUTO, gpu.TILE_AUTO, H.stream_handle())
 
 
+def test_f32_inputs_conversion_paths_agree(gpu):
+    """The conversion has a 16-byte path for aligned K-contiguous rows with K % 8 == 0 and an element-wise one for the
+    rest: the same A and B, once aligned and once starting 4 bytes into their buffers, give the same bits."""
+    M, N, K = 328, 200, 776
+    g = torch.Generator(device="cuda").manual_seed(4321)
+    a_buf = torch.randn(M * K + 4, generator=g, device="cuda", dtype=torch.float32)
+    b_buf = torch.randn(N * K + 4, generator=g, device="cuda", dtype=torch.float32)
+    a_off, b_off = a_buf[1:1 + M * K], b_buf[1:1 + N * K]          # 4 bytes past a 16-byte boundary
+    a_al, b_al = a_off.clone(), b_off.clone()
+    assert a_al.data_ptr() % 16 == 0 and a_off.data_ptr() % 16 == 4
+    out = []
+    for a, b in ((a_al, b_al), (a_off, b_off)):
+        c = H.poisoned_c(M, N)
+        t = gpu.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), gpu.F32, 0, 1, 0)
+        need = gpu.matmul_f32_workspace_bytes(t, gpu.F32_BF16X3)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        gpu.matmul_f32_ws(t, ws.data_ptr(), need, gpu.F32_BF16X3, gpu.K_OUTPUT_STATIONARY, gpu.TILE_128x128, H.stream_handle())
+        torch.cuda.synchronize()
+        out.append(c)
+    assert torch.equal(out[0], out[1])
+
+
 def test_f32_inputs_known_answer(gpu):
     """The reference's own known answer in its own element type (gemm/gemm_main.cpp:81-90, gemm/gemm_test.cu:67-72):
     tiled numbers up to 6363 times the identity.  Two bf16 terms hold every integer below 65536 exactly, so the
