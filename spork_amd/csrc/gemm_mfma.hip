@@ -826,9 +826,17 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint16_t* in, uint16_
         }
         return;
     }
-    for (uint32_t kk = ty; kk < 64; kk += 4) {
-        const uint32_t k = k0 + kk, r = r0 + tx;
-        tile[kk][tx] = (k < K && r < rows) ? in[(size_t)k * rows + r] : (uint16_t)0;
+    // (all loads of a lane in flight together: out-of-range lanes read element 0 and drop the value)
+    uint16_t v[16];
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) {
+        const uint32_t k = k0 + ty + 4 * i, r = r0 + tx;
+        v[i] = in[(k < K && r < rows) ? (size_t)k * rows + r : (size_t)0];
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) {
+        const uint32_t k = k0 + ty + 4 * i, r = r0 + tx;
+        tile[ty + 4 * i][tx] = (k < K && r < rows) ? v[i] : (uint16_t)0;
     }
     __syncthreads();
     for (uint32_t rr = ty; rr < 64; rr += 4) {
@@ -839,9 +847,56 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint16_t* in, uint16_
     }
 }
 
+// The transposing re-pack for an even number of rows and a 4-byte aligned source: 128 x 128 blocks, two elements per
+// lane on the way in (256-byte segments of a source row per wave and load, all loads of a lane in flight together),
+// eight consecutive K values (16 bytes) per lane on the way out.
+__global__ __launch_bounds__(256) void repack_transposed_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
+                                                                uint32_t rows, uint32_t K, uint32_t kp)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ uint32_t tile[128][65];  // [k][pair of rows]
+    const uint32_t r0 = blockIdx.x * 128, k0 = blockIdx.y * 128;
+    const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    const uint32_t r_in = r0 + 2 * tx;  // rows is even: a pair is inside the matrix or outside it
+    uint32_t v[32];
+#pragma unroll
+    for (uint32_t i = 0; i < 32; ++i) {
+        const uint32_t k = k0 + ty + 4 * i;
+        v[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t*>(in + ((k < K && r_in < rows) ? (size_t)k * rows + r_in : (size_t)0)));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 32; ++i) {
+        const uint32_t k = k0 + ty + 4 * i;
+        tile[ty + 4 * i][tx] = (k < K && r_in < rows) ? v[i] : 0u;
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < 128 * 16; i += 256) {
+        const uint32_t rr = i / 16, ch = i % 16;
+        const uint32_t r = r0 + rr, k = k0 + ch * 8;
+        if (r >= rows || k >= kp) {
+            continue;
+        }
+        const uint32_t shift = (rr & 1u) * 16;
+        uint32_t w[4];
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t e0 = tile[ch * 8 + 2 * j][rr / 2] >> shift & 0xffffu;
+            const uint32_t e1 = tile[ch * 8 + 2 * j + 1][rr / 2] >> shift & 0xffffu;
+            w[j] = e0 | e1 << 16;
+        }
+        *reinterpret_cast<u32x4*>(out + (size_t)r * kp + k) = u32x4{w[0], w[1], w[2], w[3]};
+    }
+}
+
 static int repack(const Operand& op, uint32_t K, void* dst, hipStream_t stream)
 {
     const uint32_t kp = (uint32_t)round_up(K, 8);
+    if (!op.k_contiguous && op.rows % 2 == 0 && (uintptr_t)op.ptr % 4 == 0) {
+        hipLaunchKernelGGL(repack_transposed_kernel, dim3((op.rows + 127) / 128, (kp + 127) / 128, 1), dim3(256), 0, stream,
+                           (const uint16_t*)op.ptr, (uint16_t*)dst, op.rows, K, kp);
+        MI_CHECK_LAUNCH();
+        return MI_OK;
+    }
     const dim3 grid((kp + 63) / 64, (op.rows + 63) / 64, 1);
     if (grid.y > 65535u) {
         return MI_ERR_UNSUPPORTED;
@@ -927,9 +982,18 @@ __global__ __launch_bounds__(256) void split_f32_transposed_kernel(const float* 
     // consecutive workgroups take neighbouring segments of the same 128 source rows
     const uint32_t r0 = blockIdx.x * 64, k0 = blockIdx.y * 128;
     const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;
-    for (uint32_t kk = ty; kk < 128; kk += 4) {
-        const uint32_t k = k0 + kk, r = r0 + tx;
-        tile[kk][tx] = (k < K && r < rows) ? __builtin_nontemporal_load(in + (size_t)k * rows + r) : 0.0f;
+    // every load is issued before the first is awaited: out-of-range lanes read element 0 and drop the value
+    float v[32];
+    const uint32_t r_in = r0 + tx;
+#pragma unroll
+    for (uint32_t i = 0; i < 32; ++i) {
+        const uint32_t k = k0 + ty + 4 * i;
+        v[i] = __builtin_nontemporal_load(in + ((k < K && r_in < rows) ? (size_t)k * rows + r_in : (size_t)0));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 32; ++i) {
+        const uint32_t k = k0 + ty + 4 * i;
+        tile[ty + 4 * i][tx] = (k < K && r_in < rows) ? v[i] : 0.0f;
     }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i < 64 * 16; i += 256) {
