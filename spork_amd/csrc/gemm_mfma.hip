@@ -708,7 +708,20 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* parti
             const T v3 = __builtin_nontemporal_load(src + (size_t)(s + 3) * count + i);
             acc = (((acc + v0) + v1) + v2) + v3;
         }
-        for (; s < splits; ++s) {
+        // the last one to three copies: loaded together, added in the same order
+        const uint32_t rest = splits - s;
+        if (rest == 3) {
+            const T v0 = __builtin_nontemporal_load(src + (size_t)s * count + i);
+            const T v1 = __builtin_nontemporal_load(src + (size_t)(s + 1) * count + i);
+            const T v2 = __builtin_nontemporal_load(src + (size_t)(s + 2) * count + i);
+            acc = ((acc + v0) + v1) + v2;
+        }
+        else if (rest == 2) {
+            const T v0 = __builtin_nontemporal_load(src + (size_t)s * count + i);
+            const T v1 = __builtin_nontemporal_load(src + (size_t)(s + 1) * count + i);
+            acc = (acc + v0) + v1;
+        }
+        else if (rest == 1) {
             acc += __builtin_nontemporal_load(src + (size_t)s * count + i);
         }
         dst[i] = acc;
