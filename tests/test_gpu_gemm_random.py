@@ -88,3 +88,45 @@ def test_random_small_problems_against_the_device_baseline(gpu, seed):
 def test_random_large_ragged_problems_against_the_device_baseline(gpu):
     plans = [_run_case(gpu, case) for case in _cases(7, 24, big=True)]
     assert sum(p not in ("unsupported", "needs workspace") for p in plans) >= 12
+
+
+def _xgemm_cases(seed, count):
+    rng = random.Random(seed)
+    out = []
+    for _ in range(count):
+        k_splits = rng.choice([1, 1, 2, 3, 5])
+        cluster_k = rng.choice([rng.randint(1, 300), 8 * rng.randint(1, 60)])
+        out.append((rng.choice([1, 1, 2, 3, 7]), rng.randint(1, 700), rng.randint(1, 700), k_splits, cluster_k,
+                    rng.choice(["F32_BF16X3", "F32_BF16X3", "F32_BF16X1"])))
+    return out
+
+
+@pytest.mark.parametrize("case", _xgemm_cases(7, 40), ids=lambda c: "L%dx%dx%dx(%dx%d)_%s" % c)
+def test_random_xgemm_argument_lists(gpu, case):
+    """Random shapes (any M, N, cluster_k; L problems; K splits) through the entry points with the reference's Exo
+    argument lists (xgemm_Sm90.py:43-48, xgemm_Sm80.py:18-21) against numpy's float64 product of the same fp32 values; C
+    starts as NaN and the workspace ends in a poisoned band."""
+    L, M, N, k_splits, cluster_k, precision = case
+    K = k_splits * cluster_k
+    prec = getattr(gpu, precision)
+    tol = 3e-5 if precision == "F32_BF16X3" else 1.5e-2
+    g = torch.Generator(device="cuda").manual_seed(L * 1000003 + M * 1009 + N * 13 + K)
+    a = torch.randn((L, M, K), generator=g, device="cuda", dtype=torch.float32)
+    b = torch.randn((L, N, K), generator=g, device="cuda", dtype=torch.float32)
+    c = torch.full((L, N, M), float("nan"), dtype=torch.float32, device="cuda")
+    need = gpu.xgemm_workspace_bytes(L, M, N, K, prec)
+    ws = torch.full((need + 512,), 0xAB, dtype=torch.uint8, device="cuda")
+    ctxt = gpu.XgemmContext(ws.data_ptr(), need, H.stream_handle(), prec, gpu.TILE_AUTO)
+    gpu.xgemm_Sm90_wgmma(ctxt, L, M, N, k_splits, cluster_k, a.data_ptr(), b.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    assert bool((ws[need:] == 0xAB).all()), "wrote past the workspace"
+    ref = np.einsum("lnk,lmk->lnm", b.cpu().numpy().astype(np.float64), a.cpu().numpy().astype(np.float64))
+    scale = max(np.abs(ref).max(), 1e-300)
+    assert np.nanmax(np.abs(c.cpu().numpy() - ref)) / scale < tol and not torch.isnan(c).any()
+    if L == 1:
+        b_rows = b[0].t().contiguous()  # K x N, as the Sm80 proc takes it
+        c2 = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        gpu.xgemm_Sm80(ctxt, M, N, K, a.data_ptr(), b_rows.data_ptr(), c2.data_ptr())
+        torch.cuda.synchronize()
+        assert bool((ws[need:] == 0xAB).all()), "wrote past the workspace"
+        assert np.nanmax(np.abs(c2.cpu().numpy() - ref[0].T)) / scale < tol and not torch.isnan(c2).any()
