@@ -69,6 +69,50 @@ def test_entry_points_replay_correctly_from_a_graph(gpu, name):
             np.testing.assert_array_equal(got, want, err_msg=f"{name} replay {replay}")
 
 
+@pytest.mark.parametrize("k_splits", [1, 3])
+def test_xgemm_entry_replays_correctly_from_a_graph(gpu, k_splits):
+    """The fp32 entry point with the reference's Exo argument list (xgemm_Sm90.py:43-48): two conversion kernels, for
+    K splits a fill kernel, and one batched GEMM launch, captured once and replayed on changing inputs."""
+    L, M, N, cluster_k = 3, 200, 264, 256
+    K = k_splits * cluster_k
+    a = torch.empty((L, M, K), dtype=torch.float32, device="cuda")
+    b = torch.empty((L, N, K), dtype=torch.float32, device="cuda")
+    c_graph = torch.empty((L, N, M), dtype=torch.float32, device="cuda")
+    c_eager = torch.empty_like(c_graph)
+    need = gpu.xgemm_workspace_bytes(L, M, N, K, gpu.F32_BF16X3)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    def call(c):
+        # (the context names the stream: torch captures on a stream of its own, current only inside the capture)
+        ctxt = gpu.XgemmContext(ws.data_ptr(), need, H.stream_handle(), gpu.F32_BF16X3, gpu.TILE_128x128)
+        gpu.xgemm_Sm90_wgmma(ctxt, L, M, N, k_splits, cluster_k, a.data_ptr(), b.data_ptr(), c.data_ptr())
+
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a.normal_(generator=g)
+    b.normal_(generator=g)
+    call(c_graph)                # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(c_graph)
+    for replay in range(4):
+        a.normal_(generator=g)
+        b.normal_(generator=g)
+        c_graph.view(torch.uint8).fill_(0x7D)
+        ws.fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        call(c_eager)
+        torch.cuda.synchronize()
+        got, want = c_graph.cpu().numpy(), c_eager.cpu().numpy()
+        assert np.isfinite(got).all(), replay
+        if k_splits > 1:
+            assert H.rel_err(got, want.astype(np.float64)) < 1e-5, replay   # atomics: the order of additions varies
+        else:
+            np.testing.assert_array_equal(got, want, err_msg=f"replay {replay}")
+
+
 _PREPARED_CAPTURE = r"""
 import sys
 import numpy as np
