@@ -1,6 +1,7 @@
 """Seeded random differential test: random shapes, layouts, dtypes, K modes, tiles and workspace sizes through the C
 ABI against the on-device baseline kernel (itself pinned against the oracle elsewhere).  C and the workspace sit inside
 poisoned guard bands so that a store outside either is caught; C starts as NaN so that an element never written is too."""
+import os
 import random
 
 import numpy as np
@@ -77,7 +78,12 @@ def _run_case(gpu, case):
     return what
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3])
+# MI_GEMM_FUZZ_SEEDS=n widens the sweep to n seeds of each kind (120 small or 24 large cases per seed; a few thousand small
+# cases take seconds)
+_SEEDS = int(os.environ.get("MI_GEMM_FUZZ_SEEDS", "0"))
+
+
+@pytest.mark.parametrize("seed", list(range(1, max(_SEEDS, 20) + 1)))
 def test_random_small_problems_against_the_device_baseline(gpu, seed):
     ran = 0
     for case in _cases(seed, 120, big=False):
@@ -85,8 +91,9 @@ def test_random_small_problems_against_the_device_baseline(gpu, seed):
     assert ran >= 60
 
 
-def test_random_large_ragged_problems_against_the_device_baseline(gpu):
-    plans = [_run_case(gpu, case) for case in _cases(7, 24, big=True)]
+@pytest.mark.parametrize("seed", list(range(7, 7 + max(_SEEDS, 4))))
+def test_random_large_ragged_problems_against_the_device_baseline(gpu, seed):
+    plans = [_run_case(gpu, case) for case in _cases(seed, 24, big=True)]
     assert sum(p not in ("unsupported", "needs workspace") for p in plans) >= 12
 
 
