@@ -733,3 +733,46 @@ def test_compare_tensors_matches_reference_rule(gpu, oracle):
     assert int(r[3]) == 2
     assert np.array([r[1]]).view(np.float64)[0] == np.abs(x.astype(np.float64) - y.astype(np.float64)).max()
     assert np.array([r[2]]).view(np.float64)[0] == np.abs(x).max()
+
+
+def test_host_threads_on_streams_of_their_own(gpu, oracle):
+    """Four host threads, each with its own stream and buffers, launch different problems at the same time (the calls
+    release the interpreter lock): every thread's results equal what one thread computes alone.  The library keeps no
+    state between calls apart from per-device flags, so callers need no lock of their own."""
+    import threading
+
+    problems = [(512, 384, 1024, 0, "K_AUTO"), (300, 200, 1000, 1, "K_AUTO"), (256, 256, 4096, 0, "K_SPLIT_REDUCE"),
+                (1024, 128, 2048, 1, "K_OUTPUT_STATIONARY")]
+    setups = []
+    for M, N, K, dtype, k_mode in problems:
+        a, b = H.make_inputs(M, N, K, dtype, 3, 3, 1.0)
+        c_alone, c_threaded = H.poisoned_c(M, N), H.poisoned_c(M, N)
+        t_alone, t_threaded = H.tensors(M, N, K, a, b, c_alone, dtype), H.tensors(M, N, K, a, b, c_threaded, dtype)
+        _, pref = gpu.matmul_mfma_workspace_bytes_for(t_alone, getattr(gpu, k_mode), gpu.TILE_AUTO)
+        ws = torch.empty(max(pref, 256), dtype=torch.uint8, device="cuda")
+        gpu.matmul_mfma_ws(t_alone, ws.data_ptr(), pref, getattr(gpu, k_mode), gpu.TILE_AUTO, H.stream_handle())
+        setups.append((t_threaded, ws, pref, getattr(gpu, k_mode), c_alone, c_threaded, a, b))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(setup):
+        try:
+            t, ws, pref, k_mode, _, c_threaded, _, _ = setup
+            stream = torch.cuda.Stream()
+            for _ in range(50):
+                gpu.matmul_mfma_ws(t, ws.data_ptr(), pref, k_mode, gpu.TILE_AUTO, stream.cuda_stream)
+            stream.synchronize()
+        except Exception as e:  # noqa: BLE001 - reported below, in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in setups]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(60)
+    assert not errors and not any(th.is_alive() for th in threads), errors
+    torch.cuda.synchronize()
+    for (t, ws, pref, k_mode, c_alone, c_threaded, a, b), (M, N, K, dtype, _) in zip(setups, problems):
+        assert torch.equal(c_alone, c_threaded), (M, N, K)
+        ref = oracle.gemm_f64(M, N, K, H.to_host_u16(a), H.to_host_u16(b), dtype)
+        assert H.rel_err(c_threaded.cpu().numpy(), ref) < TOL
