@@ -60,6 +60,17 @@ def test_vendor_library_exports_its_header():
     assert os.path.isfile(path) and "hipblaslt" in os.path.basename(path), path
 
 
+def test_headers_are_plain_c(tmp_path):
+    """The boundary is a C ABI: both public headers compile as strict C99 on their own."""
+    src = tmp_path / "abi.c"
+    src.write_text('#include "mi_gemm.h"\n#include "mi_gemm_vendor.h"\n'
+                   "int main(void) { mi_gemm_tensors t; mi_xgemm_context x; (void)t; (void)x; return 0; }\n")
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", include, "-c", str(src), "-o",
+                        str(tmp_path / "abi.o")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
 def test_struct_layout_matches_the_header():
     # uint32 x3, three pointers (8-aligned after 12 bytes -> offset 16), four uint8, padded to 8
     assert S.GpuTensors.M.offset == 0 and S.GpuTensors.K.offset == 8
