@@ -233,3 +233,39 @@ def test_operand_read_once_is_streamed_non_temporal(gpu, oracle, case):
         gpu.matmul_mfma(t2, gpu.K_OUTPUT_STATIONARY, gpu.TILE_128x128, H.stream_handle())
         torch.cuda.synchronize()
         assert float((c2 - c).abs().max()) / scale < 1e-5
+
+
+@pytest.mark.parametrize("entry", ["sm90", "sm80"])
+def test_fp32_entry_points_at_the_headline_size(gpu, entry):
+    """The Exo-named fp32 entry points (xgemm_Sm90.py:43-48 as the harness calls it, gemm/gemm_test.cu:335; xgemm_Sm80.py:18-21)
+    at 8192^3 on normal(0,1)/sqrt(K) fp32 data: Freivalds' identity C x = A (B x) over the whole matrix in float64 for
+    four random +-1 vectors, and sampled rows against numpy's float64 product, at the three-term bar (3e-5 of the
+    scale: each operand carries 16 significant bits)."""
+    M = N = K = 8192
+    g = torch.Generator(device="cuda").manual_seed(8192)
+    a = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32) * K ** -0.5
+    b_nk = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32) * K ** -0.5   # B stored N x K
+    c = H.poisoned_c(M, N)
+    need = gpu.xgemm_workspace_bytes(1, M, N, K, gpu.F32_BF16X3)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ctxt = gpu.XgemmContext(ws.data_ptr(), need, H.stream_handle(), gpu.F32_BF16X3, gpu.TILE_AUTO)
+    if entry == "sm90":
+        # operands swapped, so that the proc's C[L,N,M] is the row-major M x N
+        gpu.xgemm_Sm90_wgmma(ctxt, 1, N, M, 1, K, b_nk.data_ptr(), a.data_ptr(), c.data_ptr())
+    else:
+        b_kn = b_nk.t().contiguous()
+        gpu.xgemm_Sm80(ctxt, M, N, K, a.data_ptr(), b_kn.data_ptr(), c.data_ptr())
+        del b_kn
+    torch.cuda.synchronize()
+    ha, hb, hc = a.cpu().numpy(), b_nk.cpu().numpy(), c.cpu().numpy()
+    assert np.isfinite(hc).all()
+    rng = np.random.default_rng(11)
+    x = rng.choice([-1.0, 1.0], size=(N, 4))
+    bx = hb.astype(np.float64).T @ x                                                                # K x 4
+    want = ha.astype(np.float64) @ bx                                                               # M x 4
+    got = hc.astype(np.float64) @ x
+    scale = np.abs(ha).astype(np.float64) @ (np.abs(hb).astype(np.float64).T @ np.ones((N, 1)))      # sum |a||b| per row
+    assert (np.abs(got - want) / scale).max() < 3e-5
+    rows = np.unique(np.concatenate([np.arange(0, M, 256), np.arange(255, M, 256), rng.integers(0, M, 16)]))[:80]
+    ref_rows = ha[rows].astype(np.float64) @ hb.astype(np.float64).T
+    assert np.abs(hc[rows] - ref_rows).max() / np.abs(ref_rows).max() < 3e-5
