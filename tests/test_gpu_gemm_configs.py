@@ -269,3 +269,64 @@ def test_fp32_entry_points_at_the_headline_size(gpu, entry):
     rows = np.unique(np.concatenate([np.arange(0, M, 256), np.arange(255, M, 256), rng.integers(0, M, 16)]))[:80]
     ref_rows = ha[rows].astype(np.float64) @ hb.astype(np.float64).T
     assert np.abs(hc[rows] - ref_rows).max() / np.abs(ref_rows).max() < 3e-5
+
+
+@pytest.mark.parametrize("shape", [(70_000, 256, 32_768), (33_000, 33_000, 64), (256, 70_000, 32_768), (47_000, 47_000, 64)])
+def test_operands_and_results_beyond_four_gigabytes(gpu, shape):
+    """A of 4.6 GB, C of 4.4 GB, B of 4.6 GB, C of 2.2e9 elements: byte offsets past 2^32 in the panel bases and in C, element
+    indices past 2^31.  Checked on the device in
+    float64 (torch is the independent implementation here): Freivalds' identity over the whole matrix, and the rows at
+    the far end of the large tensor against a direct product."""
+    M, N, K = shape
+    dtype = 1
+    a = H.gen_on_device(M, K, 4, False, dtype, K ** -0.5, SEED_A)
+    b = H.gen_on_device(N, K, 4, True, dtype, K ** -0.5, SEED_B)
+    assert max(a.numel() * 2, b.numel() * 2, M * N * 4) > 1 << 32
+    c = H.run_mfma(M, N, K, a, b, dtype)
+    af, bf = a.view(torch.bfloat16), b.view(torch.bfloat16)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = (torch.randint(0, 2, (N, 4), generator=g, device="cuda") * 2 - 1).double()
+    bx = bf.double().T @ x if N * K <= 1 << 28 else torch.cat([bf[:, k0:k0 + 4096].double().T @ x for k0 in range(0, K, 4096)])
+    b_abs = bf.double().abs().sum(0) if N * K <= 1 << 28 else torch.cat([bf[:, k0:k0 + 4096].double().abs().sum(0) for k0 in range(0, K, 4096)])
+    worst = 0.0
+    for r0 in range(0, M, 2048):
+        rows = slice(r0, min(M, r0 + 2048))
+        want = af[rows].double() @ bx
+        got = c[rows].double() @ x
+        scale = af[rows].double().abs() @ b_abs
+        worst = max(worst, float(((got - want).abs().max(1).values / scale).max()))
+    assert worst < 1e-4, worst
+    for r in (0, M // 2, M - 257, M - 1):
+        ref = af[r].double() @ bf.double().T if N * K <= 1 << 28 else torch.cat([af[r].double() @ bf[n0:n0 + 4096].double().T for n0 in range(0, N, 4096)])
+        assert float((c[r].double() - ref).abs().max() / ref.abs().max()) < TOL, r
+    del a, b, c
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("k_mode", ["K_SPLIT", "K_SPLIT_REDUCE"])
+def test_k_partitions_of_a_result_beyond_four_gigabytes(gpu, k_mode):
+    """C of 4.4 GB with K partitions forced: the zero fill, the atomic epilogue, the partitions' copies of C in a
+    workspace of two or more times that size and the pass that sums them all index past 2^32 bytes."""
+    M, N, K, dtype = 33_000, 33_000, 1024, 1
+    a = H.gen_on_device(M, K, 4, False, dtype, K ** -0.5, SEED_A)
+    b = H.gen_on_device(N, K, 4, True, dtype, K ** -0.5, SEED_B)
+    c = H.poisoned_c(M, N)
+    t = H.tensors(M, N, K, a, b, c, dtype)
+    mode = getattr(gpu, k_mode)
+    plan = gpu.matmul_mfma_plan(t, mode, gpu.TILE_256x256)
+    assert plan["k_splits"] >= 2, plan
+    if k_mode == "K_SPLIT":
+        gpu.matmul_mfma(t, mode, gpu.TILE_256x256, H.stream_handle())
+    else:
+        required, preferred = gpu.matmul_mfma_workspace_bytes_for(t, mode, gpu.TILE_256x256)
+        assert required >= 2 * M * N * 4
+        ws = torch.empty(preferred, dtype=torch.uint8, device="cuda")
+        gpu.matmul_mfma_ws(t, ws.data_ptr(), preferred, mode, gpu.TILE_256x256, H.stream_handle())
+    torch.cuda.synchronize()
+    af, bf = a.view(torch.bfloat16).double(), b.view(torch.bfloat16).double()
+    worst = 0.0
+    for r0 in list(range(0, M, 4096)) + [M - 300]:
+        rows = slice(r0, min(M, r0 + 300))
+        ref = af[rows] @ bf.T
+        worst = max(worst, float((c[rows].double() - ref).abs().max() / ref.abs().max()))
+    assert worst < TOL, worst
