@@ -330,3 +330,37 @@ def test_k_partitions_of_a_result_beyond_four_gigabytes(gpu, k_mode):
         ref = af[rows] @ bf.T
         worst = max(worst, float((c[rows].double() - ref).abs().max() / ref.abs().max()))
     assert worst < TOL, worst
+
+
+@pytest.mark.parametrize("shape", [(256, 256, (1 << 21) - 64), (64, 192, (1 << 21) - 8), (300, 130, 1_500_008)])
+def test_deepest_k_the_library_accepts(gpu, shape):
+    """K just under the library's bound of 2^21 (rows of 4 MB: the largest buffer offsets a tile's DMA forms), whole
+    tiles and ragged, against torch's float64 product; K at the bound is refused."""
+    M, N, K = shape
+    dtype = 1
+    a = H.gen_on_device(M, K, 4, False, dtype, K ** -0.5, SEED_A)
+    b = H.gen_on_device(N, K, 4, True, dtype, K ** -0.5, SEED_B)
+    c = H.run_mfma(M, N, K, a, b, dtype)
+    ref = a.view(torch.bfloat16).double() @ b.view(torch.bfloat16).double().T
+    assert float((c.double() - ref).abs().max() / ref.abs().max()) < TOL
+    t = H.tensors(M, N, 1 << 21, a, b, c, dtype)
+    assert not gpu.matmul_mfma_supports(t, gpu.K_AUTO, gpu.TILE_AUTO)
+
+
+def test_deepest_k_of_the_fp32_entry(gpu):
+    """Three bf16 terms triple the depth: fp32 K = 699 048 is a bf16 problem 2 097 144 deep, the deepest accepted."""
+    M, N, K = 128, 192, 699_048
+    g = torch.Generator(device="cuda").manual_seed(21)
+    a = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32) * K ** -0.5
+    b = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32) * K ** -0.5
+    c = H.poisoned_c(M, N)
+    t = gpu.GpuTensors.make(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), gpu.F32, 0, 1, 0)
+    need = gpu.matmul_f32_workspace_bytes(t, gpu.F32_BF16X3)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    gpu.matmul_f32_ws(t, ws.data_ptr(), need, gpu.F32_BF16X3, gpu.K_AUTO, gpu.TILE_AUTO, H.stream_handle())
+    torch.cuda.synchronize()
+    ref = a.double() @ b.double().T
+    assert float((c.double() - ref).abs().max() / ref.abs().max()) < 3e-5
+    deeper = gpu.GpuTensors.make(M, N, K + 8, a.data_ptr(), b.data_ptr(), c.data_ptr(), gpu.F32, 0, 1, 0)
+    with pytest.raises(gpu.MiGemmError):
+        gpu.matmul_f32_workspace_bytes(deeper, gpu.F32_BF16X3)
