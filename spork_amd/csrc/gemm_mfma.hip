@@ -309,6 +309,15 @@ static double plan_cost(const Canonical& c, int tile, uint32_t k_splits, bool re
     else if (needs_edge(c, d)) {
         us_per_k64 *= 1.05;  // per-instruction bounds bookkeeping
     }
+    // Dense rows three times a power of two apart (K = 49152, 98304 with 16-bit elements; the HBM stacks are twelve dies
+    // high, which puts a factor of three into the address map) make the panels that workgroups fetch side by side collide
+    // in memory.  Measured against their estimates on twelve such shapes: plans of the 128-column tiles run 1.4 to 1.56
+    // times as long and the 192 x 192 tile 1.2 to 1.33 times; the 256- and 192-column tiles of 160 rows and more run
+    // 0.9 to 1.29 times as long with no pattern that a constant would capture (pricing the 256 x 256 tile up, which
+    // is off most often, only hands its problems to tiles that are hit harder), so those keep their estimates.
+    if (c.lda == c.ldb && ((uint64_t)c.lda * 2) % 98304 == 0 && c.K >= 32768) {
+        us_per_k64 *= d.bn <= 128 ? 1.45 : (d.bm == 192 && d.bn == 192) ? 1.25 : 1.0;
+    }
     const double items = (double)ceil_div(c.M, d.bm) * ceil_div(c.N, d.bn) * k_splits * c.batches;
     double waves = __builtin_ceil(items / places);
     const double k64_steps = __builtin_ceil((double)ceil_div(c.K, d.bk) / k_splits) * (d.bk / 64.0);
