@@ -126,6 +126,10 @@ def main() -> int:
     out["mfma_ceiling"] = mfma_ceiling(S, L, a if a.numel() >= b.numel() else b, dtype, stream)
     if out["mfma_ceiling"] and "value" in out["mfma_ceiling"]:
         out["roofline"]["frac_of_sustained_ceiling"] = round(achieved / out["mfma_ceiling"]["value"], 4)
+    if roofline["bound"] == "hbm":
+        out["hbm_ceiling"] = hbm_ceiling(S, L, a if a.numel() >= b.numel() else b, stream)
+        if "value" in out["hbm_ceiling"]:
+            out["roofline"]["frac_of_streaming_ceiling"] = round(roofline["achieved"] / out["hbm_ceiling"]["value"], 4)
 
     if not args.no_vendor:
         out["vendor_comparator"] = vendor_comparator(S, L, t, stream, flops, min(args.steps, 30))
@@ -151,6 +155,12 @@ def main() -> int:
                     "tflops": round(r["flops"] / (r["launch_ms"] * 1e-3) * 1e-12, 1),
                     "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
                     "max_rel_err": r["max_rel_err_vs_device_baseline"], "plan": r["roofline"]["launches"], "steps": 20}
+                if r["roofline"]["bound"] == "hbm":
+                    big = r["a"] if r["a"].numel() >= r["b"].numel() else r["b"]
+                    out["configs"][name]["hbm_ceiling"] = hbm_ceiling(S, L, big, stream)
+                    if "value" in out["configs"][name]["hbm_ceiling"]:
+                        out["configs"][name]["roofline"]["frac_of_streaming_ceiling"] = round(
+                            r["roofline"]["achieved"] / out["configs"][name]["hbm_ceiling"]["value"], 4)
             except Exception as e:  # a side measurement must never take the benchmark line down
                 out["configs"][name] = {"error": str(e)[:200]}
             r = None
@@ -322,6 +332,38 @@ def mfma_ceiling(S, L, a, dtype, stream):
         mhz = float((100.0 * h[:, 0] / h[:, 1]).mean())
         return {"value": round(flop.value / (ms.value * 1e-3) * 1e-12, 1), "unit": "TFLOP/s", "core_clock_mhz": round(mhz),
                 "what": "register-only v_mfma_f32_16x16x32 loop, one wave per SIMD on every CU, on this workload's A operand (B where B is the larger one)"}
+    except Exception as e:  # a measurement aid must never take the benchmark line down
+        return {"error": str(e)[:200]}
+
+
+def hbm_ceiling(S, L, operand, stream):
+    """What kernels that only stream this workload's large operand sustain (16-byte vector loads, the GEMM's own LDS DMA
+    with one and with two workgroups per CU, and a read-and-write copy of it): the yardstick for a memory-bound shape,
+    measured in the same process on the same buffer.  GB/s of bytes moved; median of 9 launches after 10 untimed ones."""
+    import torch
+
+    try:
+        nbytes = operand.numel() * operand.element_size()
+        dst = torch.empty_like(operand)
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        out = {"bytes": nbytes, "unit": "GB/s"}
+        for name, mode, per_cu in (("vector_loads_8_per_cu", S.STREAM_READ, 8), ("lds_dma_1_per_cu", S.STREAM_DMA, 1),
+                                   ("lds_dma_2_per_cu", S.STREAM_DMA, 2), ("copy_8_per_cu", S.STREAM_COPY, 8)):
+            def launch():
+                S.hbm_stream_ceiling(operand.data_ptr(), dst.data_ptr(), nbytes, mode, per_cu, sink.data_ptr(), stream)
+            for _ in range(10):
+                launch()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(10)]
+            ev[0].record()
+            for i in range(9):
+                launch()
+                ev[i + 1].record()
+            torch.cuda.synchronize()
+            ms = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(9))[4]
+            out[name] = round((2 if mode == S.STREAM_COPY else 1) * nbytes / (ms * 1e-3) * 1e-9, 1)
+        out["value"] = max(out["vector_loads_8_per_cu"], out["lds_dma_1_per_cu"], out["lds_dma_2_per_cu"])
+        out["what"] = "read-only streaming of this workload's largest operand; value = the best of the read-only ways"
+        return out
     except Exception as e:  # a measurement aid must never take the benchmark line down
         return {"error": str(e)[:200]}
 

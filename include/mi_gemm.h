@@ -27,6 +27,10 @@ enum {
     MI_ERR_HIP = 4,          /* a HIP runtime call failed; see mi_last_hip_error()                       */
     MI_ERR_NO_DEVICE = 5,    /* no gfx950 device visible                                                  */
 };
+/* Not every misuse has a status: two calls that use the same scratch memory while they overlap in time on one GPU - the same
+ * workspace given to mi_matmul_mfma_ws on two streams, or any two overlapping calls of mi_matmul_mfma_static or of the Exo
+ * entry points with a null context, which all share the library's one scratch array per GPU - are undefined (wrong results),
+ * and are not detected. */
 const char* mi_status_string(int status);
 /* hipError_t of the most recent failing HIP call made by this library on the calling thread (0 if none). */
 int mi_last_hip_error(void);
@@ -64,17 +68,24 @@ enum {
     MI_K_SPLIT = 1,             /* K split across workgroups; C zero-filled by the callee, partials are
                                    reduced with fp32 atomic adds (gemm/gemm_sm90.cu:1096-1115,1208-1210)  */
     MI_K_AUTO = 2,              /* library picks by shape (and by the workspace it is given)              */
-    MI_K_SPLIT_REDUCE = 3,      /* K split across workgroups; every partition stores its own copy of C in the
-                                   caller's workspace and a second kernel sums the copies in partition order:
-                                   no zero fill, no atomics, the same bits on every run.  No counterpart in the
-                                   reference (its partitions meet through TMA reduce-adds); only through
-                                   mi_matmul_mfma_ws / mi_matmul_f32_ws                                   */
-    MI_K_STREAM = 4,            /* stream-K (the role of gemm_sm90_k_mode::stream_k_*, gemm/gemm_sm90.h:10-11): one
-                                   workgroup per CU, each working an equal run of the (tile, K tile) pairs, so the
-                                   chip is full whatever the tile count; a run touches two tiles at most, its
-                                   parts go to the workspace and a second kernel sums each tile's parts in order.
-                                   For problems of whole tiles (M, N multiples of the tile, K of 64) with no more
-                                   tiles than CUs; only through mi_matmul_mfma_ws / mi_matmul_f32_ws      */
+    MI_K_SPLIT_REDUCE = 3,      /* K split across workgroups; every partition stores its own copy of its tile of C in
+                                   the caller's workspace, and the workgroup that stores a tile's last copy adds the
+                                   copies, in partition order, into C - inside the one launch, as the reference's
+                                   partitions meet in its epilogue (gemm/gemm_sm90.cu:944-963), but by plain loads and
+                                   stores in a fixed order: no zero fill, no floating-point atomics, the same bits on
+                                   every run.  (When the library's arrival counters are not to be had, see
+                                   mi_matmul_mfma_sum_in_launch, a second kernel sums the copies instead.)  Only
+                                   through mi_matmul_mfma_ws / mi_matmul_mfma_static / mi_matmul_f32_ws                 */
+    MI_K_STREAM = 4,            /* stream-K (the role of gemm_sm90_k_mode::stream_k_*, gemm/gemm_sm90.h:10-11), laid out
+                                   as gemm/gemm_sm90.cu:1009-1030 lays it out: the tiles that fill whole rounds of CUs run
+                                   output stationary; the tail tiles, fewer than a round, are split along K over one
+                                   round of workgroups (as many equal partitions per tile as fit, the K tiles left over
+                                   dealt in equal runs to the workgroups left over), so the chip is full whatever the
+                                   tile count.  Every part goes to the workspace and the workgroup that stores a tail
+                                   tile's last part adds that tile's parts in a fixed order into C: two launches (head
+                                   and tail), the same bits on every run.  For problems of whole tiles (M, N multiples
+                                   of the tile, K of 64), any tile count that is not a whole number of rounds; only
+                                   through mi_matmul_mfma_ws / mi_matmul_mfma_static / mi_matmul_f32_ws                 */
 };
 
 /* Workgroup tile family; replaces the n64/n128/n256 tile constructors (xgemm_Sm90.py:11-21,
@@ -153,6 +164,18 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
 #define MI_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream);
 
+/* Where the parts of MI_K_SPLIT_REDUCE and MI_K_STREAM are summed.  By default (1) inside the GEMM launch: the workgroup
+ * that stores a tile's last part sums the tile.  That takes one arrival counter per tile, which must be zero when the
+ * launch starts; the counters are an array inside the library's own code object (zero when it is loaded, left zero by
+ * every launch), dealt out in slabs of 4096 by workspace address: calls that share a workspace are ordered by their
+ * caller anyway and share a slab, calls on different workspaces may overlap and get slabs of their own.  A call that
+ * needs more counters than a slab holds, or finds all 256 slabs of the GPU taken by other workspaces, sums with a second
+ * kernel launch instead, as every call does after mi_matmul_mfma_sum_in_launch(0, ...).  The results are the same bits
+ * either way.  `enable` < 0 leaves the setting alone; returns the setting as it was.  *out_calls (may be NULL): how many
+ * calls of this process have summed inside their launch so far.  No reference counterpart (a diagnostic and a
+ * measurement aid: the host driver's `--kmodes` prints both). */
+int mi_matmul_mfma_sum_in_launch(int enable, uint64_t* out_calls);
+
 /* Sets up, once per device, what the first launch of a kernel would otherwise set up on the fly (the opt-in to more
  * than 64 KB of dynamic LDS, gemm/gemm_sm80.cu:473-475; the reference does it under std::call_once,
  * gemm/gemm_sm90.cu:1218-1219): every GEMM kernel that mi_matmul_mfma (workspace_bytes = 0) or mi_matmul_mfma_ws /
@@ -192,9 +215,11 @@ int mi_matmul_f32_ws(const mi_gemm_tensors* t, int precision, int k_mode, int ti
  *        C f32[L,N,M])                                                                           xgemm_Sm90.py:43-48
  * called at gemm/gemm_test.cu:288-294,326-362 (the Sm90 ones with the operands swapped, so that C[L,N,M] comes out as
  * the harness's row-major M x N).  All tensors are dense and row-major in the order written; K = K_splits * cluster_k.
- * The reference passes ctxt = nullptr, its generated code needing nothing from the caller.  This library never
- * allocates, so here ctxt brings the scratch memory the fp32 operands are converted into, and the stream (the
- * reference runs these on stream 0 only, gemm/gemm_test.cu:289,325).  K_splits > 1 selects what the reference's
+ * The reference passes ctxt = nullptr, its generated code needing nothing from the caller, and runs these on stream 0
+ * only (gemm/gemm_test.cu:289,325).  This library never allocates, so ctxt brings the scratch memory the fp32 operands
+ * are converted into, and the stream.  ctxt = NULL is the reference's call form: stream 0, MI_F32_BF16X3, MI_TILE_AUTO,
+ * and the scratch array of mi_matmul_mfma_static (MI_STATIC_SCRATCH_BYTES, shared by every such call on a GPU: calls that
+ * overlap in time race); MI_ERR_WORKSPACE when mi_xgemm_workspace_bytes(...) exceeds it (1024^3 takes 12 MiB, 8192^3 768).  K_splits > 1 selects what the reference's
  * split-K build does - C zero-filled, K partitions added into it (xgemm_Sm90.py:60-61) - with the number of
  * partitions chosen by the planner; the sum is the same.  The procs' divisibility assertions (M % 192, N % 256,
  * K % 16, cluster_k % 4) are limits of those kernels, not of the interface: every positive size is accepted.
@@ -235,8 +260,21 @@ int mi_matmul_mfma_timeline(const mi_gemm_tensors* t, int k_mode, int tile, uint
 int mi_mfma_ceiling(const void* d_operands, size_t operand_bytes, int ab_dtype, int mfma_tile, uint32_t iterations,
                     uint64_t* d_clocks, float* d_sink, uint32_t* out_workgroups, double* out_flop, void* hip_stream);
 
+/* Measurement tool, no reference counterpart: what a kernel that only streams `bytes` of d_src sustains, the yardstick for
+ * the GEMM shapes that memory bounds (mi_mfma_ceiling is the one for the shapes the matrix cores bound).
+ *   MI_STREAM_READ  16-byte non-temporal vector loads into registers (d_sink: one dword of device memory, keeps them alive);
+ *   MI_STREAM_DMA   `buffer_load_dwordx4 ... lds`, the GEMM kernel's own producer, into a ring in LDS that is never read:
+ *                   72 KB in flight per workgroup, what the 64x128 tile's four-slot ring holds ahead of the slot in use
+ *                   (bytes < 4 GiB, workgroups_per_cu <= 2);
+ *   MI_STREAM_COPY  read d_src, write d_dst (`bytes` each way): the usual copy figure.
+ * workgroups_per_cu (1..8) workgroups of 256 threads per CU; time the launch with events; rate = bytes / time (twice the
+ * bytes for MI_STREAM_COPY). */
+enum { MI_STREAM_READ = 0, MI_STREAM_DMA = 1, MI_STREAM_COPY = 2 };
+int mi_hbm_stream_ceiling(const void* d_src, void* d_dst, size_t bytes, int mode, uint32_t workgroups_per_cu,
+                          uint32_t* d_sink, void* hip_stream);
+
 /* What MI_*_AUTO resolves to for this problem when no workspace is given (for logging): fills tile, k_mode and the
- * number of K splits (1 for MI_K_STREAM). */
+ * number of K splits (1 for MI_K_STREAM, whose partitions per tail tile follow from the tile count and the CUs). */
 int mi_matmul_mfma_plan(const mi_gemm_tensors* t, int k_mode, int tile, int* out_tile, int* out_k_mode,
                         int* out_k_splits);
 /* The same as text, for a call of mi_matmul_mfma_ws with `workspace_bytes` of (aligned) workspace, 0 for

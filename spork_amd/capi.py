@@ -128,6 +128,7 @@ def lib() -> C.CDLL:
     sig("mi_matmul_mfma_timeline", i32, [tp, i32, i32, vp, u32, u32, C.POINTER(u32), vp])
     sig("mi_matmul_mfma_batched", i32, [tp, u32, C.c_uint64, C.c_uint64, C.c_uint64, i32, i32, vp])
     sig("mi_mfma_ceiling", i32, [vp, sz, i32, i32, u32, vp, vp, C.POINTER(u32), C.POINTER(C.c_double), vp])
+    sig("mi_hbm_stream_ceiling", i32, [vp, vp, sz, i32, u32, vp, vp])
     sig("mi_matmul_f32_workspace_bytes", i32, [tp, i32, C.POINTER(sz)])
     sig("mi_matmul_f32_ws", i32, [tp, i32, i32, i32, vp, sz, vp])
     xp = C.POINTER(XgemmContext)
@@ -139,6 +140,7 @@ def lib() -> C.CDLL:
     sig("mi_tile_count", i32, [])
     sig("mi_tile_shape", i32, [i32, C.POINTER(u32), C.POINTER(u32), ip, ip])
     sig("mi_matmul_mfma_prepare", i32, [tp, i32, i32, sz])
+    sig("mi_matmul_mfma_sum_in_launch", i32, [i32, C.POINTER(C.c_uint64)])
     sig("mi_k_mode_name", C.c_char_p, [i32])
     sig("mi_init_test_data", i32, [vp, u32, u32, i32, i32, i32, C.c_double, u32, vp])
     sig("mi_compare_tensors", i32, [vp, vp, u32, u32, vp, vp])
@@ -276,6 +278,24 @@ def xgemm_Sm90_wgmma(ctxt: XgemmContext | None, L: int, M: int, N: int, K_splits
     K = K_splits * cluster_k."""
     check(lib().mi_xgemm_Sm90_wgmma(C.byref(ctxt) if ctxt is not None else None, L, M, N, K_splits, cluster_k, a_ptr, b_ptr,
                                     c_ptr), "mi_xgemm_Sm90_wgmma")
+
+
+STREAM_READ, STREAM_DMA, STREAM_COPY = 0, 1, 2
+
+
+def hbm_stream_ceiling(src_ptr: int, dst_ptr: int, nbytes: int, mode: int, workgroups_per_cu: int, sink_ptr: int,
+                       stream: int = 0) -> None:
+    """One launch of the streaming probe (see mi_hbm_stream_ceiling); time it with events."""
+    check(lib().mi_hbm_stream_ceiling(src_ptr, dst_ptr, nbytes, mode, workgroups_per_cu, sink_ptr, stream),
+          "mi_hbm_stream_ceiling")
+
+
+def matmul_mfma_sum_in_launch(enable: int = -1) -> tuple[bool, int]:
+    """Where K partitions' copies and stream-K parts are summed: inside the GEMM launch (True, the default) or by a second
+    kernel.  A negative `enable` only asks.  Returns (the setting as it was, calls so far that summed inside their launch)."""
+    calls = C.c_uint64()
+    was = lib().mi_matmul_mfma_sum_in_launch(int(enable), C.byref(calls))
+    return bool(was), calls.value
 
 
 def widen_to_f32(src_ptr: int, dtype: int, dst_ptr: int, count: int, stream: int = 0) -> None:

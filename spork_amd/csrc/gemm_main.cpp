@@ -75,7 +75,7 @@ int main(int argc, char** argv)
 
     // data_style 0: all three reference styles; 1: tiled x identity; 2: identity x tiled; 3: reference random;
     // 4: uniform[-param, param]; 5: normal(0,1)/sqrt(K)
-    auto sized_tests = [&failures, &keep_bits, &out_ms, exo_rows = exo](uint32_t M, uint32_t N, uint32_t K, int data_style, int ab_dtype, double param = 1.0) {
+    auto sized_tests = [&failures, &keep_bits, &out_ms, exo_rows = exo, kmode_rows = kmodes](uint32_t M, uint32_t N, uint32_t K, int data_style, int ab_dtype, double param = 1.0) {
         TestParams params{};
         params.M = M;
         params.N = N;
@@ -104,12 +104,18 @@ int main(int argc, char** argv)
             if (matmul_mi355_supports(t, MI_K_SPLIT, MI_TILE_AUTO)) {
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k);
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k_sum);
+                if (kmode_rows) {
+                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_2);
+                }
             }
             if (matmul_mi355_supports(t, MI_K_AUTO, MI_TILE_AUTO)) {
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_auto_ws);
             }
             if (matmul_mi355_supports(t, MI_K_STREAM, MI_TILE_AUTO)) {
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_stream_k);
+                if (kmode_rows) {
+                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_stream_k_3);
+                }
             }
         }
         params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_row_major_b);  // any shape, any layout
@@ -196,7 +202,8 @@ int main(int argc, char** argv)
         }
         if (kmodes) {
             keep_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum) |
-                         algorithm_code_bit(AlgorithmCode::mi355_stream_k);
+                         algorithm_code_bit(AlgorithmCode::mi355_stream_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_2) |
+                         algorithm_code_bit(AlgorithmCode::mi355_stream_k_3);
         }
         const int style = argc > 6 ? atoi(argv[6]) : 5;
         if (style < 1 || style > 5) {

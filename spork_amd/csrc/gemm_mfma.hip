@@ -768,21 +768,8 @@ __global__ __launch_bounds__(256) void stream_k_sum_kernel(const float* parts, f
     const uint32_t t = blockIdx.x / chunks, row0 = (blockIdx.x % chunks) * 8;
     const uint32_t r = raster.sk.tiles, splits = raster.sk.splits, kr = k_tiles - raster.sk.main_k;
     const uint32_t lefts = workgroups - r * splits;
-    // leftover workgroup j owns the leftover pairs [j * units / lefts, (j + 1) * units / lefts); tile t's are
-    // [t * kr, (t + 1) * kr)
-    const uint64_t units = (uint64_t)r * kr, first = (uint64_t)t * kr, last = first + kr;
-    uint32_t j_lo = 0, j_hi = 0;  // workgroups [j_lo, j_hi) overlap the tile
-    if (lefts) {
-        j_lo = (uint32_t)(first * lefts / units);
-        j_lo = j_lo ? j_lo - 1 : 0;
-        while (j_lo < lefts && (j_lo + 1) * units / lefts <= first) {
-            ++j_lo;
-        }
-        j_hi = j_lo;
-        while (j_hi < lefts && j_hi * units / lefts < last) {
-            ++j_hi;
-        }
-    }
+    uint32_t j_lo, j_hi;  // leftover workgroups [j_lo, j_hi) overlap the tile
+    leftover_runs_of_tile(r, kr, lefts, t, j_lo, j_hi);
     uint32_t tm, tn;
     raster_tile(raster, raster.sk.first_tile + t, tm, tn);
     const uint32_t quads = bn / 4;
@@ -795,7 +782,7 @@ __global__ __launch_bounds__(256) void stream_k_sum_kernel(const float* parts, f
             acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts + (size_t)(t * splits + sp) * tile_elems + at));
         }
         for (uint32_t j = j_lo; j < j_hi; ++j) {
-            if ((uint64_t)j * units / lefts == (uint64_t)(j + 1) * units / lefts) {
+            if (leftover_run_empty(r, kr, lefts, j)) {
                 continue;  // (an empty run stores nothing)
             }
             acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts + (size_t)(r * splits + j + t) * tile_elems + at));
@@ -1084,6 +1071,73 @@ int resolve_static_scratch(void** out)
     return MI_OK;
 }
 
+// Arrival counters for launches that sum their K partitions (or stream-K parts) themselves, see GemmArgs::tile_counters.
+// They must be zero when a launch starts, and every launch leaves them zero, so they cannot live in a caller's workspace
+// (whose bytes are the caller's between calls) without a zero-fill launch per call, which would cost what the in-launch
+// sum saves.  They are a device array of the library's code object instead: zero when the code object is loaded, one copy
+// per GPU.  The array is dealt out in slabs by workspace: calls that share a workspace are already ordered by their
+// caller (they would overwrite each other's parts otherwise), so they can share a slab; calls with different workspaces
+// may overlap in time and get different slabs.  A workspace keeps its slab until the process ends (a captured graph may
+// replay the call at any time).  When all slabs are taken, or a call needs more counters than a slab holds, the call
+// sums with a second launch, as it always could.
+constexpr uint32_t COUNTER_SLABS = 256, SLAB_COUNTERS = 4096;
+static __device__ __align__(256) uint32_t tile_counter_pool[COUNTER_SLABS * SLAB_COUNTERS];
+
+static std::atomic<bool> sum_in_launch{true};
+static std::atomic<uint64_t> calls_summed_in_launch{0};
+
+static uint32_t* tile_counters_for(const void* workspace, uint64_t needed)
+{
+    if (!sum_in_launch.load(std::memory_order_relaxed)) {
+        return nullptr;
+    }
+    constexpr int MAX_DEVICES = 64;
+    struct PerDevice {
+        uint32_t* pool = nullptr;
+        const void* owner[COUNTER_SLABS] = {};
+        uint32_t used = 0;
+    };
+    static std::mutex guard;
+    static PerDevice devices[MAX_DEVICES];
+    int dev = 0;
+    if (workspace == nullptr || needed == 0 || needed > SLAB_COUNTERS || hipGetDevice(&dev) != hipSuccess || dev < 0 ||
+        dev >= MAX_DEVICES) {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(guard);
+    PerDevice& d = devices[dev];
+    if (d.pool == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(tile_counter_pool)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        d.pool = static_cast<uint32_t*>(ptr);
+    }
+    for (uint32_t i = 0; i < d.used; ++i) {
+        if (d.owner[i] == workspace) {
+            return d.pool + (size_t)i * SLAB_COUNTERS;
+        }
+    }
+    if (d.used == COUNTER_SLABS) {
+        return nullptr;
+    }
+    d.owner[d.used] = workspace;
+    return d.pool + (size_t)(d.used++) * SLAB_COUNTERS;
+}
+
+int resolve_tile_counters()
+{
+    int dev = 0;
+    MI_HIP_TRY(hipGetDevice(&dev));
+    // (looks the array's address up for this device; the slab of the library's own scratch array is claimed on the way)
+    void* scratch_ptr = nullptr;
+    if (const int st = resolve_static_scratch(&scratch_ptr)) {
+        return st;
+    }
+    return !sum_in_launch.load() || tile_counters_for(scratch_ptr, 1) != nullptr ? MI_OK : MI_ERR_HIP;
+}
+
 struct TimelineRequest {
     unsigned long long* d_stamps;
     uint32_t slots, max_workgroups;
@@ -1098,8 +1152,11 @@ struct BatchRequest {
 
 // `attributes_only`: go through the plan this call would run and set the attributes of every GEMM kernel it would
 // launch, launching nothing (mi_matmul_mfma_prepare).  The helper kernels (fill, re-pack, sums) need no attribute.
+// `workspace_owner`: the start of the caller's workspace when `workspace` is only what an earlier pass has left of it (the
+// arrival counters of a call are dealt out by workspace, see tile_counters_for); null: `workspace` itself.
 static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* workspace, size_t workspace_bytes, void* hip_stream,
-                    const TimelineRequest* timeline = nullptr, const BatchRequest* batch = nullptr, bool attributes_only = false)
+                    const TimelineRequest* timeline = nullptr, const BatchRequest* batch = nullptr, bool attributes_only = false,
+                    const void* workspace_owner = nullptr)
 {
     if (const int st = check_modes(t, k_mode, tile)) {
         return st;
@@ -1202,8 +1259,16 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         k.c = (float*)((char*)workspace + partial_off);
         k.stream_k_workgroups = sk.g;
         k.sk = stream_k_shape(sk);
+        // the workgroup that stores a tail tile's last part sums the tile (one counter per tail tile); without
+        // counters a last launch does the summing
+        k.tile_counters = attributes_only ? nullptr : tile_counters_for(workspace_owner ? workspace_owner : workspace, sk.r);
+        k.c_final = c.c;
+        k.ldc_final = c.ldc;
         const int st = launch_tile(t->ab_dtype, k, plan, stream);
-        return st || attributes_only ? st : stream_k_sum(k.c, c, sk, stream);
+        if (st == MI_OK && k.tile_counters != nullptr) {
+            calls_summed_in_launch.fetch_add(1, std::memory_order_relaxed);
+        }
+        return st || attributes_only || k.tile_counters != nullptr ? st : stream_k_sum(k.c, c, sk, stream);
     }
     if (plan.k_mode == MI_K_SPLIT_REDUCE) {
         // partition s of problem l stores its copy of C at partials[l][s]; the sum then writes the caller's C
@@ -1211,8 +1276,20 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         k.c = (float*)((char*)workspace + partial_off);
         k.c_split_bytes = (uint64_t)c.M * c.N * 4;
         k.c_batch_bytes = k.c_split_bytes * plan.k_splits;
+        // the workgroup that stores a tile's last copy sums the tile (one counter per tile of every problem); without
+        // counters a second launch does the summing
+        TileDims d;
+        tile_dims(plan.tile, c.K, d);
+        const uint64_t tiles = (uint64_t)ceil_div(c.M, d.bm) * ceil_div(c.N, d.bn) * c.batches;
+        k.tile_counters = attributes_only ? nullptr : tile_counters_for(workspace_owner ? workspace_owner : workspace, tiles);
+        k.c_final = c.c;
+        k.ldc_final = c.ldc;
+        k.c_final_batch_bytes = c.c_batch_bytes;
         const int st = launch_tile(t->ab_dtype, k, plan, stream);
-        return st || attributes_only ? st : reduce_partials(k.c, c, plan.k_splits, stream);
+        if (st == MI_OK && k.tile_counters != nullptr) {
+            calls_summed_in_launch.fetch_add(1, std::memory_order_relaxed);
+        }
+        return st || attributes_only || k.tile_counters != nullptr ? st : reduce_partials(k.c, c, plan.k_splits, stream);
     }
     if (plan.k_splits > 1 && !attributes_only) {
         // partial sums are atomically added: C must start at zero (gemm/gemm_sm90.cu:1208-1210).  A fill kernel,
@@ -1445,12 +1522,25 @@ static int run_f32(const mi_gemm_tensors* t, uint32_t batches, int precision, in
     if (const int st = check_modes(&f.bf16, k_mode, tile)) {
         return st;
     }
-    // refuse before converting anything if the bf16 problem itself cannot run
+    // Refuse before converting anything if the bf16 problem itself cannot run with what the call will give it: the K
+    // partitions' copies of C get what the converted operands leave of the workspace, and nothing when problems are batched.
+    const size_t used = round_up(f.ws_bytes, 256);
+    const size_t partial_space = batches > 1 || workspace_bytes <= used ? 0 : workspace_bytes - used;
     {
-        const Prepared p = prepare(f.bf16);
+        Prepared p = prepare(f.bf16);
+        p.c.batches = batches;
+        if (batches > 1) {
+            p.c.a_batch_bytes = (uint64_t)t->M * f.bf16.K * 2;
+            p.c.b_batch_bytes = (uint64_t)t->N * f.bf16.K * 2;
+            p.c.c_batch_bytes = (uint64_t)t->M * t->N * 4;
+        }
         Plan plan;
-        if (p.ws_bytes > 0 || !make_plan(p.c, k_mode, tile, SIZE_MAX, plan)) {
+        if (p.ws_bytes > 0) {
             return MI_ERR_UNSUPPORTED;
+        }
+        if (!make_plan(p.c, k_mode, tile, partial_space, plan)) {
+            const bool needs_room = k_mode == MI_K_SPLIT_REDUCE || k_mode == MI_K_STREAM;
+            return needs_room && make_plan(p.c, k_mode, tile, SIZE_MAX, plan) ? MI_ERR_WORKSPACE : MI_ERR_UNSUPPORTED;
         }
     }
     hipStream_t stream = as_stream(hip_stream);
@@ -1464,14 +1554,19 @@ static int run_f32(const mi_gemm_tensors* t, uint32_t batches, int precision, in
         uint32_t lo_mask;
     } ops[2] = {{t->a, const_cast<void*>(f.bf16.a), t->M, !t->a_col_major, a_lo_mask},
                 {t->b, const_cast<void*>(f.bf16.b), t->N, t->b_col_major != 0, b_lo_mask}};
+    auto aligned_rows = [&](const auto& op) { return op.k_contiguous && t->K % 8 == 0 && (uintptr_t)op.src % 16 == 0; };
     for (const auto& op : ops) {
-        if (((uint64_t)batches * op.rows + 63) / 64 > 65535u) {
+        // (only the element-by-element kernel puts the rows into grid.y; the other two have no such limit)
+        if (op.k_contiguous && !aligned_rows(op) && ((uint64_t)batches * op.rows + 63) / 64 > 65535u) {
+            return MI_ERR_UNSUPPORTED;
+        }
+        if ((uint64_t)batches * op.rows > 0xffffffffull) {
             return MI_ERR_UNSUPPORTED;
         }
     }
     for (const auto& op : ops) {
         const uint32_t rows = batches * op.rows;
-        if (op.k_contiguous && t->K % 8 == 0 && (uintptr_t)op.src % 16 == 0) {
+        if (aligned_rows(op)) {
             const uint64_t chunks = (uint64_t)rows * (t->K / 8);
             const uint64_t blocks = (chunks + 255) / 256;
             hipLaunchKernelGGL(split_f32_rows_kernel, dim3((uint32_t)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream,
@@ -1495,9 +1590,9 @@ static int run_f32(const mi_gemm_tensors* t, uint32_t batches, int precision, in
         return run_mfma(&f.bf16, k_mode, tile, nullptr, 0, hip_stream, nullptr, &req);
     }
     // what the converted operands leave of the workspace may hold K partitions' copies of C
-    const size_t used = round_up(f.ws_bytes, 256);
     if (workspace_bytes > used) {
-        return run_mfma(&f.bf16, k_mode, tile, (char*)d_workspace + used, workspace_bytes - used, hip_stream);
+        return run_mfma(&f.bf16, k_mode, tile, (char*)d_workspace + used, workspace_bytes - used, hip_stream, nullptr, nullptr, false,
+                        d_workspace);
     }
     return run_mfma(&f.bf16, k_mode, tile, nullptr, 0, hip_stream);
 }
@@ -1549,32 +1644,62 @@ int mi_xgemm_workspace_bytes(int L, int M, int N, int K, int precision, size_t* 
     return MI_OK;
 }
 
+// The reference's harness passes ctxt = nullptr (gemm/gemm_test.cu:326,335) and runs on stream 0.  A null context here
+// means the same call form: stream 0, MI_F32_BF16X3, MI_TILE_AUTO, and the library-resident scratch array of
+// mi_matmul_mfma_static for the converted operands (MI_ERR_WORKSPACE when they do not fit it).
+static int resolve_xgemm_context(const mi_xgemm_context* ctxt, const mi_gemm_tensors& t, uint32_t batches, mi_xgemm_context& out)
+{
+    if (ctxt != nullptr) {
+        out = *ctxt;
+        return MI_OK;
+    }
+    // (sizes first, so that a problem that cannot fit is refused before any device call)
+    F32Prepared f;
+    if (const int st = prepare_f32(&t, MI_F32_BF16X3, f, batches)) {
+        return st;
+    }
+    if (f.ws_bytes > STATIC_SCRATCH_BYTES) {
+        return MI_ERR_WORKSPACE;
+    }
+    void* ptr = nullptr;
+    if (const int st = resolve_static_scratch(&ptr)) {
+        return st;
+    }
+    out = mi_xgemm_context{ptr, STATIC_SCRATCH_BYTES, nullptr, MI_F32_BF16X3, MI_TILE_AUTO};
+    return MI_OK;
+}
+
 int mi_xgemm_Sm80(const mi_xgemm_context* ctxt, int M, int N, int K, const float* A, const float* B, float* C)
 {
     mi_gemm_tensors t;
-    if (!ctxt) {
-        return MI_ERR_BAD_ARGUMENT;
-    }
+    mi_xgemm_context cx;
     if (const int st = xgemm_tensors(M, N, K, A, B, C, false, false, t)) {
         return st;
     }
-    return run_f32(&t, 1, ctxt->precision, MI_K_AUTO, ctxt->tile, ctxt->d_workspace, ctxt->workspace_bytes, ctxt->hip_stream);
+    if (const int st = resolve_xgemm_context(ctxt, t, 1, cx)) {
+        return st;
+    }
+    return run_f32(&t, 1, cx.precision, MI_K_AUTO, cx.tile, cx.d_workspace, cx.workspace_bytes, cx.hip_stream);
 }
 
 int mi_xgemm_Sm90_wgmma(const mi_xgemm_context* ctxt, int L, int M, int N, int K_splits, int cluster_k, const float* A,
                         const float* B, float* C)
 {
     mi_gemm_tensors t;
-    if (!ctxt || L <= 0 || K_splits <= 0 || cluster_k <= 0) {
+    mi_xgemm_context cx;
+    if (L <= 0 || K_splits <= 0 || cluster_k <= 0) {
         return MI_ERR_BAD_ARGUMENT;
     }
     if (const int st = xgemm_tensors(M, N, (int64_t)K_splits * cluster_k, A, B, C, true, true, t)) {
         return st;
     }
+    if (const int st = resolve_xgemm_context(ctxt, t, (uint32_t)L, cx)) {
+        return st;
+    }
     // K_splits > 1 is the reference's split-K build, which zero-fills C and lets the K tasks add into it
     // (xgemm_Sm90.py:60-61,65): the same request here, with the number of partitions left to the planner
-    return run_f32(&t, (uint32_t)L, ctxt->precision, K_splits > 1 ? MI_K_SPLIT : MI_K_AUTO, ctxt->tile, ctxt->d_workspace,
-                   ctxt->workspace_bytes, ctxt->hip_stream);
+    return run_f32(&t, (uint32_t)L, cx.precision, K_splits > 1 ? MI_K_SPLIT : MI_K_AUTO, cx.tile, cx.d_workspace,
+                   cx.workspace_bytes, cx.hip_stream);
 }
 
 int mi_matmul_mfma_workspace_bytes(const mi_gemm_tensors* t, size_t* out_bytes)
@@ -1663,6 +1788,15 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
     return run_mfma(t, k_mode, tile, d_workspace, d_workspace ? workspace_bytes : 0, hip_stream);
 }
 
+int mi_matmul_mfma_sum_in_launch(int enable, uint64_t* out_calls)
+{
+    const bool was = enable < 0 ? sum_in_launch.load() : sum_in_launch.exchange(enable != 0);
+    if (out_calls) {
+        *out_calls = calls_summed_in_launch.load();
+    }
+    return was ? 1 : 0;
+}
+
 int mi_matmul_mfma_prepare(const mi_gemm_tensors* t, int k_mode, int tile, size_t workspace_bytes)
 {
     if (const int st = check_modes(t, k_mode, tile)) {
@@ -1673,6 +1807,9 @@ int mi_matmul_mfma_prepare(const mi_gemm_tensors* t, int k_mode, int tile, size_
     void* const stand_in = workspace_bytes ? reinterpret_cast<void*>(uintptr_t(256)) : nullptr;
     if (workspace_bytes && prepare(*t).ws_bytes > workspace_bytes) {
         return MI_ERR_WORKSPACE;
+    }
+    if (workspace_bytes) {
+        (void)resolve_tile_counters();  // (an address look-up that the captured call then need not make)
     }
     return run_mfma(t, k_mode, tile, stand_in, workspace_bytes, nullptr, nullptr, nullptr, true);
 }

@@ -42,6 +42,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 typedef __attribute__((address_space(3))) char lds_char;
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
 typedef const __attribute__((address_space(1))) char global_char;
 
 struct GemmArgs {
@@ -71,6 +72,16 @@ struct GemmArgs {
         uint32_t splits;      // S = workgroups / tiles: main partitions per tile, all tiles' partition s walked in step
         uint32_t main_k;      // Km: K tiles of every tile that the main partitions cover ([s*Km/S, (s+1)*Km/S) each)
     } sk;
+    // K partitions summed inside the launch (null: not).  Otherwise the launch stores parts of output tiles (the K
+    // partitions' copies of C, c_split_bytes != 0, or the parts of a stream-K launch) and the workgroup that stores the
+    // last part of a tile adds that tile's parts, in their fixed order, and writes the tile of `c_final` (row pitch
+    // `ldc_final` floats, problem l at c_final + l * c_final_batch_bytes).  tile_counters[l * tiles + tile] counts the
+    // parts of a tile that have been stored; it is zero before the launch and the workgroup that finds it complete sets
+    // it back to zero.  (Role of the reduce-adding epilogue of gemm/gemm_sm90.cu:944-963.)
+    uint32_t* tile_counters;
+    float* c_final;
+    uint32_t ldc_final;
+    uint64_t c_final_batch_bytes;
     // Diagnostic timeline (null in normal use): workgroup g writes stamp i to timeline[(g * timeline_slots + i) * 2]
     // (the 100 MHz constant clock) and [.. + 1] (the core clock counter): kernel entry, then per work item the point where
     // K tile 0 has landed, the end of its K loop and the end of its epilogue issue, then the point where all of the
@@ -166,7 +177,9 @@ __device__ __forceinline__ uint32_t pinned_add(uint32_t s, uint32_t v)
 // into M0 one gap ahead (base + a constant in one scalar add; the write needs a wait state before a DMA may use it,
 // which the MFMA in between provides), the
 // DMA itself names a descriptor held in four scalar registers.  The compiler does not know that M0 is live between the
-// two: the loops that use them contain no other user of M0 (checked in the ISA by the code generation test).
+// two: the code between them contains no other writer of M0 (checked in every tile's listing by the code generation test,
+// which finds the two halves by the comments they carry: every `dma-issue` must find, as the last write of M0 before it
+// in the listing, a `dma-base`, with an MFMA or a wait state in between).
 // (M0 is on the clobber list so that the compiler re-initialises it before any LDS DMA of its own that follows, e.g.
 // the ring fill of a stream-K workgroup's next part; clang remarks that M0 is a reserved register, which is the point.)
 #pragma clang diagnostic push
@@ -175,10 +188,10 @@ template <int IMM>
 __device__ __forceinline__ void dma_set_lds_base(uint32_t lds_addr)
 {
     if constexpr (IMM == 0) {
-        asm volatile("s_mov_b32 m0, %0" ::"s"(lds_addr) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0 ; dma-base" ::"s"(lds_addr) : "memory", "m0");
     }
     else {
-        asm volatile("s_add_i32 m0, %0, %1" ::"s"(lds_addr), "n"(IMM) : "memory", "m0", "scc");
+        asm volatile("s_add_i32 m0, %0, %1 ; dma-base" ::"s"(lds_addr), "n"(IMM) : "memory", "m0", "scc");
     }
 }
 #pragma clang diagnostic pop
@@ -186,10 +199,10 @@ template <bool NONTEMPORAL>
 __device__ __forceinline__ void dma_issue_16B(u32x4 rsrc, uint32_t voffset, uint32_t soffset)
 {
     if constexpr (NONTEMPORAL) {
-        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen nt lds" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen nt lds ; dma-issue" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
     }
     else {
-        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+        asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds ; dma-issue" ::"v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
     }
 }
 // Descriptor words for [base, base + bytes), as make_rsrc builds them
@@ -249,6 +262,130 @@ template <int N>
 __device__ __forceinline__ void wait_lgkmcnt()
 {
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
+}
+
+// Stream-K: the leftover workgroups [j_lo, j_hi) whose runs overlap tail tile t.  Leftover workgroup j owns the
+// leftover (tile, K tile) pairs [j * units / lefts, (j + 1) * units / lefts), units = tiles * kr; tile t's pairs are
+// [t * kr, (t + 1) * kr).  (A run may be empty when there are more leftover workgroups than pairs: see leftover_run_empty.)
+__device__ __forceinline__ void leftover_runs_of_tile(uint32_t tiles, uint32_t kr, uint32_t lefts, uint32_t t, uint32_t& j_lo,
+                                                      uint32_t& j_hi)
+{
+    j_lo = j_hi = 0;
+    if (lefts == 0) {
+        return;
+    }
+    const uint64_t units = (uint64_t)tiles * kr, first = (uint64_t)t * kr, last = first + kr;
+    j_lo = (uint32_t)(first * lefts / units);
+    j_lo = j_lo ? j_lo - 1 : 0;
+    while (j_lo < lefts && (j_lo + 1) * units / lefts <= first) {
+        ++j_lo;
+    }
+    j_hi = j_lo;
+    while (j_hi < lefts && j_hi * units / lefts < last) {
+        ++j_hi;
+    }
+}
+__device__ __forceinline__ bool leftover_run_empty(uint32_t tiles, uint32_t kr, uint32_t lefts, uint32_t j)
+{
+    const uint64_t units = (uint64_t)tiles * kr;
+    return (uint64_t)j * units / lefts == (uint64_t)(j + 1) * units / lefts;
+}
+
+// A workgroup has stored one part of an output tile: make the part visible to the whole device, count it, and tell
+// every thread of the workgroup whether it was the tile's last part (the counter is then set back to zero, for the next
+// launch: nobody else touches it any more in this one).  Nobody waits for anybody.  `lds_flag`: a dword of LDS that no one
+// is using.  The device-scope release writes this XCD's L2 back (the XCDs' L2s are private), the acquire drops what this
+// one may hold of the other parts' addresses from an earlier launch.
+__device__ __forceinline__ bool part_stored_is_it_the_last(uint32_t* counter, uint32_t expected, volatile lds_u32* lds_flag)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = before + 1 == expected;
+        if (last) {
+            __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        *lds_flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    const bool last = *lds_flag != 0u;
+    if (last) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    return last;
+}
+
+// C tile = part(0) + part(1) + ... + part(n_parts - 1), added in that order (so the result does not depend on which
+// workgroup does the adding, or when).  part(i) is where element (0, 0) of the tile lies in part i; every part has row
+// pitch `ld_part`.  T = f32x4: every pointer and pitch is a multiple of 16 bytes and columns come four at a time; T =
+// float otherwise.  Rows from `m_rem` and columns from `n_rem` on do not exist.  All parts of U places of a thread are
+// requested before the first is awaited (up to four parts at a time): a lone workgroup has only its own loads in flight
+// to cover the memory latency with.  (U = 8 takes about 160 vector registers.)
+template <int BM, int BN, int NTHREADS, typename T, uint32_t U, typename PartFn>
+__device__ __forceinline__ void sum_tile_parts(PartFn part, uint32_t n_parts, uint32_t ld_part, float* c_tile, uint32_t ldc,
+                                               int32_t m_rem, int32_t n_rem)
+{
+    constexpr uint32_t W = sizeof(T) / 4, Q = BN / W, TOTAL = BM * Q;
+    for (uint32_t first = threadIdx.x; first < TOTAL; first += NTHREADS * U) {
+        uint32_t at_part[U], at_c[U];
+        bool exists[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t idx = first + u * NTHREADS, row = idx / Q, col = (idx % Q) * W;
+            exists[u] = idx < TOTAL && (int32_t)row < m_rem && (int32_t)col < n_rem;
+            // (a place that does not exist reads element (0, 0), which does, and stores nothing)
+            at_part[u] = exists[u] ? row * ld_part + col : 0u;
+            at_c[u] = row * ldc + col;
+        }
+        T acc[U];
+        const float* const p0 = part(0);
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            acc[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(p0 + at_part[u]));
+        }
+        uint32_t i = 1;
+        for (; i + 2 < n_parts; i += 3) {
+            const float* const q0 = part(i), * const q1 = part(i + 1), * const q2 = part(i + 2);
+            T v0[U], v1[U], v2[U];
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                v0[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
+                v1[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q1 + at_part[u]));
+                v2[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q2 + at_part[u]));
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                acc[u] = ((acc[u] + v0[u]) + v1[u]) + v2[u];
+            }
+        }
+        if (i + 1 < n_parts) {
+            const float* const q0 = part(i), * const q1 = part(i + 1);
+            T v0[U], v1[U];
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                v0[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
+                v1[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q1 + at_part[u]));
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                acc[u] = (acc[u] + v0[u]) + v1[u];
+            }
+        }
+        else if (i < n_parts) {
+            const float* const q0 = part(i);
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                acc[u] += __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            if (exists[u]) {
+                __builtin_nontemporal_store(acc[u], reinterpret_cast<T*>(c_tile + at_c[u]));
+            }
+        }
+    }
 }
 
 // Tile configuration.  BK is the K depth of one ring slot; WM x WN waves tile the BM x BN block.
@@ -460,6 +597,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         const char* b_base;
         float* c_tile;                // where element (0, 0) of this item's output tile goes
         int32_t m_rem, n_rem, k_rem;  // rows of A, rows of B and K elements that exist from this item's origin on
+        // parts summed inside the launch (p.tile_counters != null): the tile's arrival counter, how many parts it has,
+        // this part's place in their order, and where the tile's sum goes
+        uint32_t counter, parts, part_index;
+        float* final_tile;
     };
     auto make_item = [&](uint32_t id) {
         Item it;
@@ -474,6 +615,11 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         it.m_rem = (int32_t)(p.M - it.tm * BM);
         it.n_rem = (int32_t)(p.N - it.tn * BN);
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
+        it.counter = batch * (p.tiles_m * p.tiles_n) + it.tm * p.tiles_n + it.tn;
+        it.parts = p.k_splits;
+        it.part_index = split;
+        it.final_tile = (float*)((char*)p.c_final + batch * p.c_final_batch_bytes) +
+                        ((size_t)it.tm * BM * p.ldc_final + (size_t)it.tn * BN);
         // (short ranges are not rotated: the walk's look-ahead must stay inside one lap)
         it.rot = EDGE || it.KT < 16 ? 0u : ((blockIdx.x % NUM_XCD) * p.k_rotate) % it.KT;
         return it;
@@ -531,6 +677,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
         it.n_rem = BN;
         it.k_rem = (int32_t)(p.K - kt_begin * BK);
         it.rot = 0;
+        it.counter = tile;
+        it.part_index = tile;  // (stream-K: the tail tile; the parts' order is their slots')
+        it.parts = 0;          // (counted when the part has been stored)
+        it.final_tile = p.c_final + ((size_t)it.tm * BM * p.ldc_final + (size_t)it.tn * BN);
         return it;
     };
     Item cur;
@@ -658,8 +808,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             break;  // (a leftover workgroup whose run is empty)
         }
         if (!first_part) {
-            // every wave has drained its fragment reads of the previous part (lgkmcnt(0) below): the ring may be refilled
-            asm volatile("s_barrier" ::: "memory");
+            // every wave has drained its fragment reads of the previous part (lgkmcnt(0) below): the ring may be refilled.
+            // (The full wait: the K loop counts its fragment reads with partial waits, and no scalar load that the code
+            // behind the previous part's K loop may have issued can be allowed to still be in flight then.)
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
         cur = make_part();
     }
@@ -1126,6 +1278,63 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                                                                       inside ? voff + soff : OOB, 0u, NT);
                             }
                         }
+                    }
+                }
+            }
+        }
+
+        if constexpr (!ATOMIC) {
+            if (p.tile_counters != nullptr) {
+                // This was one part of its tile (a K partition's copy, or a stream-K part).  Whoever stores a tile's last
+                // part adds them all up, in their fixed order, into the caller's C.
+                volatile lds_u32* const flag = (volatile lds_u32*)(lds_char*)smem;  // (the ring is no longer in use)
+                // places per thread in flight: fewer for a tile that shares its CU with a second workgroup, which has
+                // half of the registers
+                constexpr uint32_t SUM_U = 2 * Cfg::LDS_BYTES <= 160 * 1024 ? 4 : 8;
+                if constexpr (STREAM) {
+                    const uint32_t tiles = p.sk.tiles, S = p.sk.splits, lefts = gridDim.x - tiles * S, t = cur.part_index;
+                    uint32_t j_lo, j_hi, left_parts = 0;
+                    leftover_runs_of_tile(tiles, sk_kr, lefts, t, j_lo, j_hi);
+                    for (uint32_t j = j_lo; j < j_hi; ++j) {
+                        left_parts += leftover_run_empty(tiles, sk_kr, lefts, j) ? 0u : 1u;
+                    }
+                    if (part_stored_is_it_the_last(p.tile_counters + cur.counter, S + left_parts, flag)) {
+                        // main partitions' slots t * S ..., then the leftover workgroups' slots tiles * S + j + t
+                        auto part = [&](uint32_t i) -> const float* {
+                            uint32_t slot = t * S + i;
+                            if (i >= S) {
+                                uint32_t j = j_lo;
+                                for (uint32_t skip = i - S;; ++j) {
+                                    if (!leftover_run_empty(tiles, sk_kr, lefts, j)) {
+                                        if (skip == 0) {
+                                            break;
+                                        }
+                                        --skip;
+                                    }
+                                }
+                                slot = tiles * S + j + t;
+                            }
+                            return p.c + (size_t)slot * (BM * BN);
+                        };
+                        const bool vec = p.ldc_final % 4u == 0 && ((uintptr_t)cur.final_tile & 15u) == 0;
+                        if (vec) {
+                            sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
+                        }
+                        else {
+                            sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
+                        }
+                    }
+                }
+                else if (part_stored_is_it_the_last(p.tile_counters + cur.counter, cur.parts, flag)) {
+                    const char* const part0 = (const char*)cur.c_tile - (size_t)cur.part_index * p.c_split_bytes;
+                    auto part = [&](uint32_t i) -> const float* { return (const float*)(part0 + (size_t)i * p.c_split_bytes); };
+                    const bool vec = p.ldc % 4u == 0 && p.ldc_final % 4u == 0 && p.c_split_bytes % 16u == 0 &&
+                                     (((uintptr_t)part0 | (uintptr_t)cur.final_tile) & 15u) == 0;
+                    if (vec) {
+                        sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
+                    }
+                    else {
+                        sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
                     }
                 }
             }

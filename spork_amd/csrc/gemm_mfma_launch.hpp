@@ -69,6 +69,12 @@ struct Canonical {
     // a plain launch over the first `first_tiles_only` tiles of the raster order only (0: all tiles): the whole rounds
     // of a problem whose last tiles run as a stream-K launch
     uint32_t first_tiles_only = 0;
+    // parts summed inside the launch (see GemmArgs::tile_counters): the arrival counters (null: not), the caller's C, its row
+    // pitch (0 = N) and its batch stride
+    uint32_t* tile_counters = nullptr;
+    float* c_final = nullptr;
+    uint32_t ldc_final = 0;
+    uint64_t c_final_batch_bytes = 0;
     // 1: A, 2: B is read once by the launch and too large to stay cached (see gemm_tn_kernel, ONCE); the launcher
     // ignores it where no such build exists
     int read_once = 0;
@@ -147,6 +153,12 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
     args.b_batch_bytes = c.b_batch_bytes;
     args.c_batch_bytes = c.c_batch_bytes;
     args.c_split_bytes = k_splits > 1 ? c.c_split_bytes : 0;
+    // (K partitions' copies of C, or stream-K parts; a sum inside the launch needs one or the other)
+    const bool sums_inside = c.tile_counters != nullptr && c.c_final != nullptr && (args.c_split_bytes != 0 || c.stream_k_workgroups > 0);
+    args.tile_counters = sums_inside ? c.tile_counters : nullptr;
+    args.c_final = c.c_final;
+    args.ldc_final = c.ldc_final ? c.ldc_final : c.N;
+    args.c_final_batch_bytes = c.c_final_batch_bytes;
     // every partition must own at least one K tile
     if ((uint64_t)args.k_tiles_per_split * (k_splits - 1) >= k_tiles) {
         return MI_ERR_UNSUPPORTED;

@@ -143,6 +143,14 @@ int gemm_test(TestParams params, gpu_stream_t stream)
               case AlgorithmCode::mi355_stream_k:
                 matmul_mi355_any_layout(t, stream_ws, MI_K_STREAM, MI_TILE_AUTO);
                 break;
+              case AlgorithmCode::mi355_split_k_sum_2:
+              case AlgorithmCode::mi355_stream_k_3: {
+                const int was = mi_matmul_mfma_sum_in_launch(0, nullptr);
+                matmul_mi355_any_layout(t, stream_ws, algo == AlgorithmCode::mi355_stream_k_3 ? MI_K_STREAM : MI_K_SPLIT_REDUCE,
+                                        MI_TILE_AUTO);
+                mi_matmul_mfma_sum_in_launch(was, nullptr);
+                break;
+              }
               // gemm/gemm_test.cu:326,335,358,362 and :288-294: the Sm90 ones with the operands swapped, so that their
               // C[L,N,M] is the row-major M x N of the harness
               case AlgorithmCode::exo_sm_80_fence: {
@@ -221,7 +229,7 @@ int gemm_test(TestParams params, gpu_stream_t stream)
         double samples_ms = 0.0;
         const int sample_count = (test_count + 1) / 2;
         for (int i = 0; i < sample_count; ++i) {
-            samples_ms += test_times[test_count / 4 + i];  // We time based on the IQR.
+            samples_ms += test_times[test_count / 4 + i];  // the middle half of the sorted samples (gemm/gemm_test.cu:399-404)
         }
         const double flops = sample_count * double(params.M) * params.N * params.K * 2.0 * 1000.0 / samples_ms;
         if (params.out_ms) {

@@ -148,9 +148,10 @@ inline void matmul_mi355_any_layout(GPU_Tensors t, StreamWorkspace& stream_ws, i
 
 // The entry points that the reference's Exo procs compile to, by their names and argument lists (proc signatures
 // xgemm_Sm80.py:18-21 and xgemm_Sm90.py:43-48, instances xgemm_Sm90_n{64,128,256}.py:3 and
-// xgemm_Sm90_n256_tma_to_gmem.py:3-4; called at gemm/gemm_test.cu:288-294,326-362).  The reference passes ctxt = nullptr;
-// here ctxt points to a mi_xgemm_context, which names the stream and the scratch memory that the fp32 operands are
-// converted into (xgemm_context below fills one from a StreamWorkspace).  The n64 / n128 / n256 instances differ in
+// xgemm_Sm90_n256_tma_to_gmem.py:3-4; called at gemm/gemm_test.cu:288-294,326-362).  The reference passes ctxt = nullptr,
+// which is accepted here too and means stream 0 and the library's own 64 MiB scratch array for the converted fp32
+// operands (problems whose converted operands do not fit it end in MI_ERR_WORKSPACE).  Otherwise ctxt points to a
+// mi_xgemm_context, which names the stream and the scratch memory (xgemm_context below fills one from a StreamWorkspace).  The n64 / n128 / n256 instances differ in
 // their tile; here each stands for the tile of this chip's family nearest to it, unless ctxt->tile names one.  The
 // fence and mbarrier builds of the Sm80 proc, and the plain and tma_to_gmem builds of the Sm90 one, differ in how the
 // kernel synchronises and stores, not in what is computed: they are one call each here.
@@ -176,7 +177,9 @@ inline void xgemm_Sm90_wgmma_variant(const char* what, int namesake_tile, void* 
                                      int cluster_k, const float* A, const float* B, float* C)
 {
     if (!ctxt) {
-        gpu_check(MI_ERR_BAD_ARGUMENT, what);
+        // the reference's own call form (gemm/gemm_test.cu:335): stream 0, the library's resident scratch, bf16x3, any tile
+        gpu_check(mi_xgemm_Sm90_wgmma(nullptr, L, M, N, K_splits, cluster_k, A, B, C), what);
+        return;
     }
     mi_xgemm_context with_tile = *static_cast<const mi_xgemm_context*>(ctxt);
     if (with_tile.tile == MI_TILE_AUTO) {

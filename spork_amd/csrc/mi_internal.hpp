@@ -35,6 +35,10 @@ int device_compute_units();
 // device; `out` may be null).  Allocates nothing.
 int resolve_static_scratch(void** out);
 
+// Looks up, on the current device, the address of the arrival counters behind the launches that sum their K partitions
+// themselves (the first such call on a device does it otherwise).  Allocates nothing.
+int resolve_tile_counters();
+
 // Basic validation shared by every GEMM entry point: non-null, non-zero, known dtype, flags are 0/1.
 int validate_tensors(const mi_gemm_tensors* t);
 

@@ -94,6 +94,7 @@ int mi_rt_set_device(int device)
     // the set-up call of a process that uses this device: look up the address of the library's scratch array here, so
     // that mi_matmul_mfma_static finds it ready (it looks it up itself, and reports a failure, when this did not)
     (void)resolve_static_scratch(nullptr);
+    (void)resolve_tile_counters();
     return MI_OK;
 }
 

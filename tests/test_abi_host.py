@@ -367,10 +367,16 @@ def test_xgemm_entries_sizes_and_validation():
     need = S.xgemm_workspace_bytes(1, 192, 256, 64)
     ctxt = S.XgemmContext(4096, need, None, S.F32_BF16X3, S.TILE_AUTO)
     p = 4096  # placeholder addresses: every call below is refused before anything is launched
-    assert lib.mi_xgemm_Sm80(None, 192, 256, 64, p, p, p) == 2                        # the context is not optional
+    # a null context is the reference's call form (gemm/gemm_test.cu:326,335): the library's resident scratch stands in,
+    # so what does not fit its 64 MiB is refused by size, and bad sizes are refused as with a context
+    assert lib.mi_xgemm_Sm80(None, 8192, 8192, 8192, p, p, p) == 3
+    assert lib.mi_xgemm_Sm90_wgmma(None, 1, 8192, 8192, 1, 8192, p, p, p) == 3
+    assert lib.mi_xgemm_Sm90_wgmma(None, 8, 1024, 1024, 1, 1024, p, p, p) == 3         # eight problems of 12 MiB each
+    assert lib.mi_xgemm_Sm80(None, 0, 256, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm80(None, 192, 256, 64, None, p, p) == 2
     assert lib.mi_xgemm_Sm80(C.byref(ctxt), 0, 256, 64, p, p, p) == 2
     assert lib.mi_xgemm_Sm80(C.byref(ctxt), 192, 256, 64, None, p, p) == 2
-    assert lib.mi_xgemm_Sm90_wgmma(None, 1, 192, 256, 1, 64, p, p, p) == 2
+    assert lib.mi_xgemm_Sm90_wgmma(None, 0, 192, 256, 1, 64, p, p, p) == 2
     assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 0, 192, 256, 1, 64, p, p, p) == 2
     assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 1, 192, 256, 0, 64, p, p, p) == 2
     assert lib.mi_xgemm_Sm90_wgmma(C.byref(ctxt), 1, 192, 256, 1, 0, p, p, p) == 2

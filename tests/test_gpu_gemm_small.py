@@ -197,9 +197,10 @@ SUM_SHAPES = [(256, 512, 2048), (300, 500, 1000), (33, 65, 4104), (160, 480, 816
 @pytest.mark.parametrize("tile", list(range(14)))
 @pytest.mark.parametrize("shape", SUM_SHAPES)
 def test_mfma_split_k_workspace_sum(gpu, oracle, dtype, tile, shape):
-    """K partitions store private copies of C in the workspace and a second kernel sums them in partition order:
-    same accuracy bound as the atomic mode, the same bits on every run, nothing stored outside C or the workspace,
-    and an error (not a fallback) when the forced mode gets too little room."""
+    """K partitions store private copies of C in the workspace and the copies are summed in partition order, by the
+    workgroup that stores a tile's last copy (inside the launch, the default) or by a second kernel (the fallback, here
+    switched on by hand): same accuracy bound as the atomic mode, the same bits on every run and either way, nothing
+    stored outside C or the workspace, and an error (not a fallback) when the forced mode gets too little room."""
     M, N, K = shape
     a, b = H.make_inputs(M, N, K, dtype, 3, 3, 1.0)
     ref = oracle.gemm_f64(M, N, K, H.to_host_u16(a), H.to_host_u16(b), dtype)
@@ -214,17 +215,27 @@ def test_mfma_split_k_workspace_sum(gpu, oracle, dtype, tile, shape):
     ws_inner = ws[guard * 4:guard * 4 + pref]
     assert ws_inner.data_ptr() % 256 == 0
     runs = []
-    for poison in (0x7D, 0xFF):   # 0xFF bytes are NaNs: nothing of the old C or workspace may leak into the sum
+    # 0xFF bytes are NaNs: nothing of the old C or workspace may leak into the sum
+    for poison, in_launch in ((0x7D, True), (0xFF, True), (0xFF, False)):
         buf.view(torch.uint8).fill_(poison)
         ws.fill_(poison)
-        gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), pref, gpu.K_SPLIT_REDUCE, tile, H.stream_handle())
+        gpu.matmul_mfma_sum_in_launch(in_launch)
+        try:
+            calls_before = gpu.matmul_mfma_sum_in_launch()[1]
+            gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), pref, gpu.K_SPLIT_REDUCE, tile, H.stream_handle())
+            calls = gpu.matmul_mfma_sum_in_launch()[1] - calls_before
+        finally:
+            gpu.matmul_mfma_sum_in_launch(True)
         torch.cuda.synchronize()
+        # (the in-launch sum may fall back when every slab of counters is taken by other workspaces, never the reverse)
+        assert calls <= (1 if in_launch else 0)
         runs.append(c.cpu().numpy().copy())
         assert H.rel_err(runs[-1], ref) < TOL, plan
         edges = torch.cat([buf[:guard], buf[guard + M * N:]]).view(torch.uint8)
         assert bool((edges == poison).all()), "stored outside C"
         assert bool((ws[:guard * 4] == poison).all()) and bool((ws[guard * 4 + pref:] == poison).all()), "stored outside the workspace"
     np.testing.assert_array_equal(runs[0], runs[1])
+    np.testing.assert_array_equal(runs[0], runs[2])
     # the least room there is: two partitions, still inside the workspace given
     ws.fill_(0x7D)
     c.fill_(float("nan"))
@@ -295,8 +306,8 @@ STREAM_CASES = [  # (tile, bm, bn, tiles_m, tiles_n, K tiles): 4 to 5 K tiles pe
 def test_mfma_stream_k(gpu, oracle, dtype, case):
     """Stream-K: whole rounds of tiles output stationary, the tail tiles' K tiles dealt evenly to one round of
     workgroups (main partitions in step, leftover runs across tiles), parts in the workspace, summed in a fixed order by
-    a last kernel.  Same bits on every run; nothing outside C or the workspace; the forced mode refuses too small a
-    workspace."""
+    the workgroup that stores a tile's last part (or by a last kernel, the fallback, here switched on by hand).  Same bits
+    on every run and either way; nothing outside C or the workspace; the forced mode refuses too small a workspace."""
     tile_name, bm, bn, tiles_m, tiles_n, k_tiles = case
     tile = getattr(gpu, tile_name)
     M, N, K = bm * tiles_m, bn * tiles_n, 64 * k_tiles
@@ -313,10 +324,14 @@ def test_mfma_stream_k(gpu, oracle, dtype, case):
     ws = torch.empty(need + 2 * guard * 4, dtype=torch.uint8, device="cuda")
     ws_inner = ws[guard * 4:guard * 4 + need]
     runs = []
-    for poison in (0x7D, 0xFF):
+    for poison, in_launch in ((0x7D, True), (0xFF, True), (0xFF, False)):
         buf.view(torch.uint8).fill_(poison)
         ws.fill_(poison)
-        gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), need, gpu.K_STREAM, tile, H.stream_handle())
+        gpu.matmul_mfma_sum_in_launch(in_launch)
+        try:
+            gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), need, gpu.K_STREAM, tile, H.stream_handle())
+        finally:
+            gpu.matmul_mfma_sum_in_launch(True)
         torch.cuda.synchronize()
         runs.append(c.cpu().numpy().copy())
         assert H.rel_err(runs[-1], ref) < TOL, plan
@@ -324,6 +339,7 @@ def test_mfma_stream_k(gpu, oracle, dtype, case):
         assert bool((edges == poison).all()), "stored outside C"
         assert bool((ws[:guard * 4] == poison).all()) and bool((ws[guard * 4 + need:] == poison).all()), "stored outside the workspace"
     np.testing.assert_array_equal(runs[0], runs[1])
+    np.testing.assert_array_equal(runs[0], runs[2])
     with pytest.raises(gpu.MiGemmError):
         gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), need - 1, gpu.K_STREAM, tile, H.stream_handle())
 
@@ -642,6 +658,43 @@ def test_xgemm_sm90_as_the_harness_calls_it(gpu, oracle):
     torch.cuda.synchronize()
     ref = oracle.gemm_f64(M, N, K, a16.cpu().numpy().view("uint16").reshape(M, K), b16.cpu().numpy().view("uint16").reshape(N, K), dtype)
     assert H.rel_err(c.cpu().numpy(), ref) < 1e-5
+
+
+def test_xgemm_null_context_is_the_reference_call_form(gpu):
+    """The harness line verbatim, `xgemm_Sm90_wgmma_n256(nullptr, 1, N, M, 1, K, d_bCol, d_a, d_c)` on stream 0
+    (gemm/gemm_test.cu:335), and `xgemm_Sm80_fence(nullptr, M, N, K, d_a, d_b, d_c)` (:326): a null context means stream 0,
+    bf16x3 and the library's resident scratch array.  1024^3 (12 MiB of converted operands) against numpy's float64
+    product, twice in a row with a smaller problem second (the array keeps the last call's bytes); 8192^3 (768 MiB) is
+    refused with MI_ERR_WORKSPACE and leaves C alone."""
+    import ctypes as C
+
+    import numpy as np
+
+    lib = gpu.lib()
+    g = torch.Generator(device="cuda").manual_seed(335)
+    for M, N, K in ((1024, 1024, 1024), (320, 200, 136)):
+        a = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32)
+        b_col = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32)   # B stored N x K: the harness's d_bCol
+        c = H.poisoned_c(M, N)
+        torch.cuda.synchronize()
+        gpu.xgemm_Sm90_wgmma(None, 1, N, M, 1, K, b_col.data_ptr(), a.data_ptr(), c.data_ptr())
+        torch.cuda.synchronize()
+        ha, hb = a.cpu().numpy().astype(np.float64), b_col.cpu().numpy().astype(np.float64)
+        assert H.rel_err(c.cpu().numpy(), ha @ hb.T) < 3e-5, (M, N, K)
+        b_rows = b_col.t().contiguous()                                               # K x N row-major: the harness's d_b
+        c2 = H.poisoned_c(M, N)
+        torch.cuda.synchronize()
+        gpu.xgemm_Sm80(None, M, N, K, a.data_ptr(), b_rows.data_ptr(), c2.data_ptr())
+        torch.cuda.synchronize()
+        assert H.rel_err(c2.cpu().numpy(), ha @ hb.T) < 3e-5, (M, N, K)
+    big = 8192
+    assert gpu.xgemm_workspace_bytes(1, big, big, big) > gpu.STATIC_SCRATCH_BYTES
+    before = c.clone()
+    p = c.data_ptr()  # (refused before any operand is touched: the addresses only have to be non-null)
+    assert lib.mi_xgemm_Sm90_wgmma(None, 1, big, big, 1, big, p, p, p) == 3
+    assert lib.mi_xgemm_Sm80(None, big, big, big, p, p, p) == 3
+    torch.cuda.synchronize()
+    assert torch.equal(c, before)
 
 
 @pytest.mark.parametrize("tile", [16, 32])

@@ -127,6 +127,7 @@ failures = 0
 cases = {"output_stationary": (512, 768, 1024, S.K_OUTPUT_STATIONARY, S.TILE_256x256, 0),
          "split_k_workspace_sum": (256, 384, 4096, S.K_SPLIT_REDUCE, S.TILE_128x128, 1 << 24),
          "ragged_edge_build": (300, 504, 1000, S.K_AUTO, S.TILE_AUTO, 0),
+         "stream_k": (256, 768, 21888, S.K_STREAM, S.TILE_256x256, 80 << 20),
          "static_scratch": (256, 384, 4096, S.K_SPLIT_REDUCE, S.TILE_64x128, -1)}
 for name, (M, N, K, k_mode, tile, ws_bytes) in cases.items():
     a, b = H.dev_u16(M, K), H.dev_u16(N, K)
@@ -161,6 +162,9 @@ for name, (M, N, K, k_mode, tile, ws_bytes) in cases.items():
         same = np.array_equal(c_graph.cpu().numpy().view(np.uint32), c_eager.cpu().numpy().view(np.uint32))
         print(f"{name} replay {replay}: {'same bits' if same else 'DIFFERENT'}", flush=True)
         failures += not same
+# the three calls with a workspace summed their parts inside the launch, captured (once) and eager (three times)
+print(f"in-launch sums: {S.matmul_mfma_sum_in_launch()[1]}", flush=True)
+failures += S.matmul_mfma_sum_in_launch()[1] != 3 * 4
 sys.exit(1 if failures else 0)
 """
 
@@ -176,4 +180,4 @@ def test_capture_preceded_only_by_prepare(gpu):
     out = subprocess.run([sys.executable, "-c", _PREPARED_CAPTURE, root], capture_output=True, text=True, timeout=110)
     print(out.stdout[-3000:], out.stderr[-3000:], flush=True)
     assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
-    assert out.stdout.count("same bits") == 12
+    assert out.stdout.count("same bits") == 15
