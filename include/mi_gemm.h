@@ -69,23 +69,23 @@ enum {
                                    reduced with fp32 atomic adds (gemm/gemm_sm90.cu:1096-1115,1208-1210)  */
     MI_K_AUTO = 2,              /* library picks by shape (and by the workspace it is given)              */
     MI_K_SPLIT_REDUCE = 3,      /* K split across workgroups; every partition stores its own copy of its tile of C in
-                                   the caller's workspace, and the workgroup that stores a tile's last copy adds the
-                                   copies, in partition order, into C - inside the one launch, as the reference's
-                                   partitions meet in its epilogue (gemm/gemm_sm90.cu:944-963), but by plain loads and
-                                   stores in a fixed order: no zero fill, no floating-point atomics, the same bits on
-                                   every run.  (When the library's arrival counters are not to be had, see
-                                   mi_matmul_mfma_sum_in_launch, a second kernel sums the copies instead.)  Only
-                                   through mi_matmul_mfma_ws / mi_matmul_mfma_static / mi_matmul_f32_ws                 */
+                                   the caller's workspace and the copies are added in partition order into C: no zero
+                                   fill, no floating-point atomics, the same bits on every run.  By a second kernel, or
+                                   (mi_matmul_mfma_sum_in_launch) inside the one launch by the workgroup that stores a
+                                   tile's last copy, as the reference's partitions meet in its epilogue
+                                   (gemm/gemm_sm90.cu:944-963).  Only through mi_matmul_mfma_ws / mi_matmul_mfma_static /
+                                   mi_matmul_f32_ws                                                                   */
     MI_K_STREAM = 4,            /* stream-K (the role of gemm_sm90_k_mode::stream_k_*, gemm/gemm_sm90.h:10-11), laid out
                                    as gemm/gemm_sm90.cu:1009-1030 lays it out: the tiles that fill whole rounds of CUs run
                                    output stationary; the tail tiles, fewer than a round, are split along K over one
                                    round of workgroups (as many equal partitions per tile as fit, the K tiles left over
                                    dealt in equal runs to the workgroups left over), so the chip is full whatever the
-                                   tile count.  Every part goes to the workspace and the workgroup that stores a tail
-                                   tile's last part adds that tile's parts in a fixed order into C: two launches (head
-                                   and tail), the same bits on every run.  For problems of whole tiles (M, N multiples
-                                   of the tile, K of 64), any tile count that is not a whole number of rounds; only
-                                   through mi_matmul_mfma_ws / mi_matmul_mfma_static / mi_matmul_f32_ws                 */
+                                   tile count.  Every part goes to the workspace and each tail tile's parts are added in
+                                   a fixed order into C, by a last kernel or (mi_matmul_mfma_sum_in_launch) by the
+                                   workgroup that stores the tile's last part: the same bits on every run.  For problems
+                                   of whole tiles (M, N multiples of the tile, K of 64), any tile count that is not a
+                                   whole number of rounds; only through mi_matmul_mfma_ws / mi_matmul_mfma_static /
+                                   mi_matmul_f32_ws                                                                   */
 };
 
 /* Workgroup tile family; replaces the n64/n128/n256 tile constructors (xgemm_Sm90.py:11-21,
@@ -164,16 +164,20 @@ int mi_matmul_mfma_ws(const mi_gemm_tensors* t, int k_mode, int tile, void* d_wo
 #define MI_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* hip_stream);
 
-/* Where the parts of MI_K_SPLIT_REDUCE and MI_K_STREAM are summed.  By default (1) inside the GEMM launch: the workgroup
- * that stores a tile's last part sums the tile.  That takes one arrival counter per tile, which must be zero when the
- * launch starts; the counters are an array inside the library's own code object (zero when it is loaded, left zero by
- * every launch), dealt out in slabs of 4096 by workspace address: calls that share a workspace are ordered by their
- * caller anyway and share a slab, calls on different workspaces may overlap and get slabs of their own.  A call that
- * needs more counters than a slab holds, or finds all 256 slabs of the GPU taken by other workspaces, sums with a second
- * kernel launch instead, as every call does after mi_matmul_mfma_sum_in_launch(0, ...).  The results are the same bits
- * either way.  `enable` < 0 leaves the setting alone; returns the setting as it was.  *out_calls (may be NULL): how many
- * calls of this process have summed inside their launch so far.  No reference counterpart (a diagnostic and a
- * measurement aid: the host driver's `--kmodes` prints both). */
+/* Where the parts of MI_K_SPLIT_REDUCE and MI_K_STREAM are summed: by a kernel launch of its own behind the GEMM (0, the
+ * default), or inside the GEMM launch (1), where the workgroup that stores a tile's last part adds the tile's parts - the
+ * reference's scheme (gemm/gemm_sm90.cu:944-963,1004-1095), with plain loads and stores in a fixed order in place of its
+ * reduce-adds.  The results are the same bits either way.  The default is the faster way on MI355X on every shape measured
+ * (2048 x 2048 x 65536 in four partitions: 404 against 434 us; 160 x 480 x 816 in seven: 7.4 against 21 us): making a part
+ * visible to the other XCDs and dropping stale lines takes device-wide cache operations of about 15 us per launch, and only
+ * one workgroup per tile sums where the extra launch puts every CU to it.
+ * The sum inside the launch takes one arrival counter per tile, zero when the launch starts; the counters are an array in
+ * the library's own code object (zero when it is loaded, left zero by every launch), dealt out in slabs of 4096 by
+ * workspace address: calls that share a workspace are ordered by their caller anyway and share a slab, calls on different
+ * workspaces may overlap and get slabs of their own.  A call that needs more counters than a slab holds, or finds all 256
+ * slabs of the GPU taken by other workspaces, sums with the extra launch.
+ * `enable` < 0 leaves the setting alone; returns the setting as it was.  *out_calls (may be NULL): how many calls of this
+ * process have summed inside their launch so far.  The host driver's `--kmodes` prints both ways. */
 int mi_matmul_mfma_sum_in_launch(int enable, uint64_t* out_calls);
 
 /* Sets up, once per device, what the first launch of a kernel would otherwise set up on the fly (the opt-in to more
@@ -272,6 +276,12 @@ int mi_mfma_ceiling(const void* d_operands, size_t operand_bytes, int ab_dtype, 
 enum { MI_STREAM_READ = 0, MI_STREAM_DMA = 1, MI_STREAM_COPY = 2 };
 int mi_hbm_stream_ceiling(const void* d_src, void* d_dst, size_t bytes, int mode, uint32_t workgroups_per_cu,
                           uint32_t* d_sink, void* hip_stream);
+/* The same LDS DMA with the access pattern of the GEMM's tall-skinny tile on its large operand: a row-major matrix of
+ * `rows` x `row_bytes` (a multiple of 128), every workgroup walking `rows_per_workgroup` (a multiple of 8) consecutive rows
+ * 128 bytes at a time, 72 KB in flight: what the memory system gives a kernel that reads an operand panel by panel and
+ * nothing else.  One workgroup per `rows_per_workgroup` rows; rate = rows * row_bytes / time. */
+int mi_hbm_stream_rows_ceiling(const void* d_src, uint32_t rows, uint32_t row_bytes, uint32_t rows_per_workgroup,
+                               void* hip_stream);
 
 /* What MI_*_AUTO resolves to for this problem when no workspace is given (for logging): fills tile, k_mode and the
  * number of K splits (1 for MI_K_STREAM, whose partitions per tail tile follow from the tile count and the CUs). */

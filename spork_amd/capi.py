@@ -129,6 +129,7 @@ def lib() -> C.CDLL:
     sig("mi_matmul_mfma_batched", i32, [tp, u32, C.c_uint64, C.c_uint64, C.c_uint64, i32, i32, vp])
     sig("mi_mfma_ceiling", i32, [vp, sz, i32, i32, u32, vp, vp, C.POINTER(u32), C.POINTER(C.c_double), vp])
     sig("mi_hbm_stream_ceiling", i32, [vp, vp, sz, i32, u32, vp, vp])
+    sig("mi_hbm_stream_rows_ceiling", i32, [vp, u32, u32, u32, vp])
     sig("mi_matmul_f32_workspace_bytes", i32, [tp, i32, C.POINTER(sz)])
     sig("mi_matmul_f32_ws", i32, [tp, i32, i32, i32, vp, sz, vp])
     xp = C.POINTER(XgemmContext)
@@ -288,6 +289,11 @@ def hbm_stream_ceiling(src_ptr: int, dst_ptr: int, nbytes: int, mode: int, workg
     """One launch of the streaming probe (see mi_hbm_stream_ceiling); time it with events."""
     check(lib().mi_hbm_stream_ceiling(src_ptr, dst_ptr, nbytes, mode, workgroups_per_cu, sink_ptr, stream),
           "mi_hbm_stream_ceiling")
+
+
+def hbm_stream_rows_ceiling(src_ptr: int, rows: int, row_bytes: int, rows_per_workgroup: int, stream: int = 0) -> None:
+    """One launch of the LDS DMA probe with a GEMM operand panel's access pattern (see mi_hbm_stream_rows_ceiling)."""
+    check(lib().mi_hbm_stream_rows_ceiling(src_ptr, rows, row_bytes, rows_per_workgroup, stream), "mi_hbm_stream_rows_ceiling")
 
 
 def matmul_mfma_sum_in_launch(enable: int = -1) -> tuple[bool, int]:

@@ -105,7 +105,7 @@ int main(int argc, char** argv)
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k);
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k_sum);
                 if (kmode_rows) {
-                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_2);
+                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_in);
                 }
             }
             if (matmul_mi355_supports(t, MI_K_AUTO, MI_TILE_AUTO)) {
@@ -114,7 +114,7 @@ int main(int argc, char** argv)
             if (matmul_mi355_supports(t, MI_K_STREAM, MI_TILE_AUTO)) {
                 params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_stream_k);
                 if (kmode_rows) {
-                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_stream_k_3);
+                    params.algorithm_code_bits |= algorithm_code_bit(AlgorithmCode::mi355_stream_k_in);
                 }
             }
         }
@@ -202,8 +202,8 @@ int main(int argc, char** argv)
         }
         if (kmodes) {
             keep_bits |= algorithm_code_bit(AlgorithmCode::mi355_split_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum) |
-                         algorithm_code_bit(AlgorithmCode::mi355_stream_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_2) |
-                         algorithm_code_bit(AlgorithmCode::mi355_stream_k_3);
+                         algorithm_code_bit(AlgorithmCode::mi355_stream_k) | algorithm_code_bit(AlgorithmCode::mi355_split_k_sum_in) |
+                         algorithm_code_bit(AlgorithmCode::mi355_stream_k_in);
         }
         const int style = argc > 6 ? atoi(argv[6]) : 5;
         if (style < 1 || style > 5) {

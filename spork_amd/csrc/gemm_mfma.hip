@@ -1083,7 +1083,9 @@ int resolve_static_scratch(void** out)
 constexpr uint32_t COUNTER_SLABS = 256, SLAB_COUNTERS = 4096;
 static __device__ __align__(256) uint32_t tile_counter_pool[COUNTER_SLABS * SLAB_COUNTERS];
 
-static std::atomic<bool> sum_in_launch{true};
+// Off unless asked for: measured on MI355X the sum inside the launch is the slower way on every shape tried (see
+// mi_matmul_mfma_sum_in_launch in mi_gemm.h).
+static std::atomic<bool> sum_in_launch{false};
 static std::atomic<uint64_t> calls_summed_in_launch{0};
 
 static uint32_t* tile_counters_for(const void* workspace, uint64_t needed)

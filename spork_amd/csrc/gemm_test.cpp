@@ -143,10 +143,10 @@ int gemm_test(TestParams params, gpu_stream_t stream)
               case AlgorithmCode::mi355_stream_k:
                 matmul_mi355_any_layout(t, stream_ws, MI_K_STREAM, MI_TILE_AUTO);
                 break;
-              case AlgorithmCode::mi355_split_k_sum_2:
-              case AlgorithmCode::mi355_stream_k_3: {
-                const int was = mi_matmul_mfma_sum_in_launch(0, nullptr);
-                matmul_mi355_any_layout(t, stream_ws, algo == AlgorithmCode::mi355_stream_k_3 ? MI_K_STREAM : MI_K_SPLIT_REDUCE,
+              case AlgorithmCode::mi355_split_k_sum_in:
+              case AlgorithmCode::mi355_stream_k_in: {
+                const int was = mi_matmul_mfma_sum_in_launch(1, nullptr);
+                matmul_mi355_any_layout(t, stream_ws, algo == AlgorithmCode::mi355_stream_k_in ? MI_K_STREAM : MI_K_SPLIT_REDUCE,
                                         MI_TILE_AUTO);
                 mi_matmul_mfma_sum_in_launch(was, nullptr);
                 break;

@@ -26,10 +26,10 @@ enum class AlgorithmCode
     mi355_split_k,        // planner picks the tile, K split forced
     mi355_row_major_b,    // B given K x N row-major (the baseline's own call): re-packed through the workspace
     mi355_auto_ws,        // planner with a workspace at hand: K partitions may be summed from copies of C
-    mi355_split_k_sum,    // K split forced, partitions summed from copies of C in the workspace (no atomics), in the one launch
+    mi355_split_k_sum,    // K split forced, partitions summed from copies of C in the workspace (no atomics)
     mi355_stream_k,       // stream-K forced: equal runs of (tile, K tile) pairs, parts summed from the workspace
-    mi355_split_k_sum_2,  // the two rows above with the parts summed by a launch of its own instead of inside the GEMM
-    mi355_stream_k_3,     //   launch (mi_matmul_mfma_sum_in_launch(0)): only where asked for (--kmodes)
+    mi355_split_k_sum_in,  // the two rows above with the parts summed inside the GEMM launch instead of by a launch of its
+    mi355_stream_k_in,     //   own (mi_matmul_mfma_sum_in_launch(1)): only where asked for (--kmodes)
     hipblaslt,            // vendor comparator (the cuBLAS / CUTLASS rows of gemm/gemm_test.h:19-20)
     exo_sm_80_fence,      // the reference's Exo entry points by name (gemm/gemm_test.h:21-31), on the test data widened
     exo_sm_90_n256,       //   to fp32: three bf16 terms per product, so about 3.3x the 16-bit time
@@ -83,10 +83,10 @@ inline const char* algorithm_name(AlgorithmCode code)
         return "mi355 (split k, workspace sum)";
       case AlgorithmCode::mi355_stream_k:
         return "mi355 (stream k)";
-      case AlgorithmCode::mi355_split_k_sum_2:
-        return "mi355 (split k, workspace sum by a second launch)";
-      case AlgorithmCode::mi355_stream_k_3:
-        return "mi355 (stream k, sum by a third launch)";
+      case AlgorithmCode::mi355_split_k_sum_in:
+        return "mi355 (split k, workspace sum inside the launch)";
+      case AlgorithmCode::mi355_stream_k_in:
+        return "mi355 (stream k, sum inside the tail launch)";
       case AlgorithmCode::hipblaslt:
         return "hipBLASLt";
       case AlgorithmCode::exo_sm_80_fence:

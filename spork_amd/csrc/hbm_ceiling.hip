@@ -7,6 +7,8 @@
 //   MI_STREAM_DMA        `buffer_load_dwordx4 ... lds`, the GEMM kernel's own producer: 1 KB per wave instruction
 //                        straight into a ring in LDS, nothing ever read back, as many in flight as the GEMM's ring keeps;
 //   MI_STREAM_COPY       read and write back (half of the bytes each way), the usual "copy bandwidth" figure.
+// And the DMA again with the access pattern of a GEMM operand panel (mi_hbm_stream_rows_ceiling): 128-byte pieces of many
+// rows instead of contiguous kilobytes.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -91,9 +93,75 @@ __global__ __launch_bounds__(256) void stream_dma_kernel(const void* src, uint32
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// DMA_ROWS: the same ring, fed the way the GEMM's tall-skinny tile reads its A panel: workgroup g owns `rows_per_wg`
+// consecutive rows of a row-major matrix with `row_bytes` per row and walks them 128 bytes (one 64-deep K tile of 16-bit
+// elements) at a time, every DMA instruction fetching 128 bytes from each of eight rows (lane i: row i / 8 of the eight,
+// chunk i % 8).  Same bytes as DMA, same number in flight, but 128-byte pieces a whole row apart instead of contiguous 1 KB.
+// byte offset of piece p = (K tile p / groups, group of eight rows p % groups) within a workgroup's rows
+__device__ __forceinline__ uint32_t rows_piece_offset(uint32_t p, uint32_t groups, uint32_t row_bytes)
+{
+    return (p % groups) * 8u * row_bytes + (p / groups) * 128u;
+}
+
+template <int IN_FLIGHT>
+__global__ __launch_bounds__(256) void stream_dma_rows_kernel(const void* src, uint32_t rows, uint32_t row_bytes, uint32_t rows_per_wg)
+{
+    extern __shared__ __attribute__((aligned(1024))) char ring[];
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    lds_char* const mine = (lds_char*)ring + w * (IN_FLIGHT * 1024);
+    const uint32_t first_row = blockIdx.x * rows_per_wg;
+    if (first_row + rows_per_wg > rows) {
+        return;
+    }
+    // descriptor over this workgroup's rows; the lane's part of the address never changes
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>((const char*)src + (size_t)first_row * row_bytes), 0, rows_per_wg * row_bytes, 0x00020000);
+    const uint32_t voff = (lane / 8u) * row_bytes + (lane % 8u) * 16u;
+    // one K tile = rows_per_wg / 8 instructions, dealt round-robin to the four waves; piece p = (K tile, group of 8 rows)
+    const uint32_t groups = rows_per_wg / 8u, pieces = (row_bytes / 128u) * groups;
+    uint32_t piece = w;
+#pragma unroll
+    for (int s = 0; s < IN_FLIGHT; ++s) {
+        if (piece < pieces) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, mine + s * 1024, 16, voff, rows_piece_offset(piece, groups, row_bytes), 0, 0);
+        }
+        piece += 4u;
+    }
+    while (piece < pieces) {
+#pragma unroll
+        for (int s = 0; s < IN_FLIGHT; ++s) {
+            if (piece < pieces) {
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT - 1) : "memory");
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, mine + s * 1024, 16, voff, rows_piece_offset(piece, groups, row_bytes), 0, 0);
+            }
+            piece += 4u;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 }  // namespace mi_gemm
 
 using namespace mi_gemm;
+
+extern "C" int mi_hbm_stream_rows_ceiling(const void* d_src, uint32_t rows, uint32_t row_bytes, uint32_t rows_per_workgroup,
+                                          void* hip_stream)
+{
+    if (!d_src || (uintptr_t)d_src % 16 || rows == 0 || row_bytes == 0 || row_bytes % 128 || rows_per_workgroup == 0 ||
+        rows_per_workgroup % 8 || rows_per_workgroup > rows) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    if ((uint64_t)rows_per_workgroup * row_bytes >= ((uint64_t)1 << 31)) {
+        return MI_ERR_UNSUPPORTED;  // a workgroup's rows must stay within the reach of one buffer descriptor
+    }
+    constexpr int lds = 4 * 18 * 1024;
+    MI_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&stream_dma_rows_kernel<18>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    hipLaunchKernelGGL(stream_dma_rows_kernel<18>, dim3(rows / rows_per_workgroup), dim3(256), lds, as_stream(hip_stream), d_src, rows,
+                       row_bytes, rows_per_workgroup);
+    MI_CHECK_LAUNCH();
+    return MI_OK;
+}
 
 extern "C" int mi_hbm_stream_ceiling(const void* d_src, void* d_dst, size_t bytes, int mode, uint32_t workgroups_per_cu,
                                      uint32_t* d_sink, void* hip_stream)

@@ -42,7 +42,7 @@ for name, M, N, K, in_launch in cases:
     for i in range(LAUNCHES):
         S.matmul_mfma_ws(H.tensors(M, N, K, a, b, outs[i], S.BF16), ws.data_ptr(), need, S.K_STREAM, tile, st)
     torch.cuda.synchronize()
-    S.matmul_mfma_sum_in_launch(True)
+    S.matmul_mfma_sum_in_launch(False)
     differs = (outs.view(torch.int32) != outs[0].view(torch.int32)).flatten(1).any(dim=1).cpu().numpy()
     if differs.any():
         i = int(np.argmax(differs))

@@ -198,8 +198,7 @@ SUM_SHAPES = [(256, 512, 2048), (300, 500, 1000), (33, 65, 4104), (160, 480, 816
 @pytest.mark.parametrize("shape", SUM_SHAPES)
 def test_mfma_split_k_workspace_sum(gpu, oracle, dtype, tile, shape):
     """K partitions store private copies of C in the workspace and the copies are summed in partition order, by the
-    workgroup that stores a tile's last copy (inside the launch, the default) or by a second kernel (the fallback, here
-    switched on by hand): same accuracy bound as the atomic mode, the same bits on every run and either way, nothing
+    workgroup that stores a tile's last copy (inside the launch, switched on by hand) or by a second kernel (the default): same accuracy bound as the atomic mode, the same bits on every run and either way, nothing
     stored outside C or the workspace, and an error (not a fallback) when the forced mode gets too little room."""
     M, N, K = shape
     a, b = H.make_inputs(M, N, K, dtype, 3, 3, 1.0)
@@ -219,13 +218,12 @@ def test_mfma_split_k_workspace_sum(gpu, oracle, dtype, tile, shape):
     for poison, in_launch in ((0x7D, True), (0xFF, True), (0xFF, False)):
         buf.view(torch.uint8).fill_(poison)
         ws.fill_(poison)
-        gpu.matmul_mfma_sum_in_launch(in_launch)
+        was, calls_before = gpu.matmul_mfma_sum_in_launch(in_launch)
         try:
-            calls_before = gpu.matmul_mfma_sum_in_launch()[1]
             gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), pref, gpu.K_SPLIT_REDUCE, tile, H.stream_handle())
             calls = gpu.matmul_mfma_sum_in_launch()[1] - calls_before
         finally:
-            gpu.matmul_mfma_sum_in_launch(True)
+            gpu.matmul_mfma_sum_in_launch(was)
         torch.cuda.synchronize()
         # (the in-launch sum may fall back when every slab of counters is taken by other workspaces, never the reverse)
         assert calls <= (1 if in_launch else 0)
@@ -306,7 +304,7 @@ STREAM_CASES = [  # (tile, bm, bn, tiles_m, tiles_n, K tiles): 4 to 5 K tiles pe
 def test_mfma_stream_k(gpu, oracle, dtype, case):
     """Stream-K: whole rounds of tiles output stationary, the tail tiles' K tiles dealt evenly to one round of
     workgroups (main partitions in step, leftover runs across tiles), parts in the workspace, summed in a fixed order by
-    the workgroup that stores a tile's last part (or by a last kernel, the fallback, here switched on by hand).  Same bits
+    the workgroup that stores a tile's last part (switched on by hand) or by a last kernel (the default).  Same bits
     on every run and either way; nothing outside C or the workspace; the forced mode refuses too small a workspace."""
     tile_name, bm, bn, tiles_m, tiles_n, k_tiles = case
     tile = getattr(gpu, tile_name)
@@ -327,11 +325,11 @@ def test_mfma_stream_k(gpu, oracle, dtype, case):
     for poison, in_launch in ((0x7D, True), (0xFF, True), (0xFF, False)):
         buf.view(torch.uint8).fill_(poison)
         ws.fill_(poison)
-        gpu.matmul_mfma_sum_in_launch(in_launch)
+        was, _ = gpu.matmul_mfma_sum_in_launch(in_launch)
         try:
             gpu.matmul_mfma_ws(t, ws_inner.data_ptr(), need, gpu.K_STREAM, tile, H.stream_handle())
         finally:
-            gpu.matmul_mfma_sum_in_launch(True)
+            gpu.matmul_mfma_sum_in_launch(was)
         torch.cuda.synchronize()
         runs.append(c.cpu().numpy().copy())
         assert H.rel_err(runs[-1], ref) < TOL, plan

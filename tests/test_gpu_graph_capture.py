@@ -123,6 +123,7 @@ import spork_amd as S
 
 torch.cuda.set_device(0)
 failures = 0
+S.matmul_mfma_sum_in_launch(True)   # (not the default: the captured launches then carry the library's arrival counters)
 # name: (M, N, K, k_mode, tile, workspace bytes; -1: the library's own scratch array)
 cases = {"output_stationary": (512, 768, 1024, S.K_OUTPUT_STATIONARY, S.TILE_256x256, 0),
          "split_k_workspace_sum": (256, 384, 4096, S.K_SPLIT_REDUCE, S.TILE_128x128, 1 << 24),

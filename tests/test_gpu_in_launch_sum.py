@@ -1,7 +1,8 @@
 """The sum of K partitions (MI_K_SPLIT_REDUCE) and of stream-K parts (MI_K_STREAM) inside the GEMM launch: the workgroup
 that stores a tile's last part adds the tile's parts, in their fixed order, into C (the role of the reduce-adding epilogue
 of gemm/gemm_sm90.cu:944-963, with the work generators of :1004-1095).  The arrival counters behind it live in the
-library, are zero before a launch and must be zero again after it.
+library, are zero before a launch and must be zero again after it.  (The library sums with a kernel launch of its own
+unless mi_matmul_mfma_sum_in_launch switches this on: measured, that is the faster way on this chip.)
 
 The checks run in a process of their own, so that every slab of counters is free at its start and the test can tell from
 the library's call count which way a call summed."""
@@ -25,6 +26,7 @@ import spork_amd as S
 torch.cuda.set_device(0)
 st = H.stream_handle()
 failures = 0
+S.matmul_mfma_sum_in_launch(True)   # (the library's default is the sum by a launch of its own)
 
 def report(what, ok):
     global failures
