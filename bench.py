@@ -130,6 +130,8 @@ def main() -> int:
         out["hbm_ceiling"] = hbm_ceiling(S, L, a if a.numel() >= b.numel() else b, stream)
         if "value" in out["hbm_ceiling"]:
             out["roofline"]["frac_of_streaming_ceiling"] = round(roofline["achieved"] / out["hbm_ceiling"]["value"], 4)
+        if "lds_dma_rows_64_per_workgroup" in out["hbm_ceiling"]:
+            out["roofline"]["frac_of_row_pattern_ceiling"] = round(roofline["achieved"] / out["hbm_ceiling"]["lds_dma_rows_64_per_workgroup"], 4)
 
     if not args.no_vendor:
         out["vendor_comparator"] = vendor_comparator(S, L, t, stream, flops, min(args.steps, 30))
@@ -161,6 +163,9 @@ def main() -> int:
                     if "value" in out["configs"][name]["hbm_ceiling"]:
                         out["configs"][name]["roofline"]["frac_of_streaming_ceiling"] = round(
                             r["roofline"]["achieved"] / out["configs"][name]["hbm_ceiling"]["value"], 4)
+                    if "lds_dma_rows_64_per_workgroup" in out["configs"][name]["hbm_ceiling"]:
+                        out["configs"][name]["roofline"]["frac_of_row_pattern_ceiling"] = round(
+                            r["roofline"]["achieved"] / out["configs"][name]["hbm_ceiling"]["lds_dma_rows_64_per_workgroup"], 4)
             except Exception as e:  # a side measurement must never take the benchmark line down
                 out["configs"][name] = {"error": str(e)[:200]}
             r = None
@@ -361,8 +366,26 @@ def hbm_ceiling(S, L, operand, stream):
             torch.cuda.synchronize()
             ms = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(9))[4]
             out[name] = round((2 if mode == S.STREAM_COPY else 1) * nbytes / (ms * 1e-3) * 1e-9, 1)
+        # the same DMA with the access pattern of a tile's operand panel: 128-byte pieces of 64 (128) rows per workgroup
+        rows, row_bytes = operand.shape[0], operand.shape[1] * operand.element_size()
+        for per_wg in (64, 128):
+            if rows % per_wg or row_bytes % 128:
+                continue
+            def launch():
+                S.hbm_stream_rows_ceiling(operand.data_ptr(), rows, row_bytes, per_wg, stream)
+            for _ in range(10):
+                launch()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(10)]
+            ev[0].record()
+            for i in range(9):
+                launch()
+                ev[i + 1].record()
+            torch.cuda.synchronize()
+            ms = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(9))[4]
+            out[f"lds_dma_rows_{per_wg}_per_workgroup"] = round(nbytes / (ms * 1e-3) * 1e-9, 1)
         out["value"] = max(out["vector_loads_8_per_cu"], out["lds_dma_1_per_cu"], out["lds_dma_2_per_cu"])
-        out["what"] = "read-only streaming of this workload's largest operand; value = the best of the read-only ways"
+        out["what"] = ("read-only streaming of this workload's largest operand; value = the best of the contiguous read-only "
+                       "ways; lds_dma_rows_*: the DMA reading 128-byte pieces row by row, as a GEMM tile reads its panel")
         return out
     except Exception as e:  # a measurement aid must never take the benchmark line down
         return {"error": str(e)[:200]}

@@ -403,6 +403,24 @@ def test_ceiling_probe_validates_its_arguments():
     assert lib.mi_mfma_ceiling(4100, 1 << 26, S.BF16, 16, 10, 4096, 8192, C.byref(n), C.byref(f), None) == 2   # alignment
 
 
+def test_streaming_probes_validate_their_arguments():
+    lib = S.lib()
+    p = 4096
+    assert lib.mi_hbm_stream_ceiling(None, p, 1 << 20, S.STREAM_READ, 1, p, None) == 2
+    assert lib.mi_hbm_stream_ceiling(p + 4, p, 1 << 20, S.STREAM_READ, 1, p, None) == 2      # alignment
+    assert lib.mi_hbm_stream_ceiling(p, p, 512, S.STREAM_READ, 1, p, None) == 2              # too few bytes
+    assert lib.mi_hbm_stream_ceiling(p, p, 1 << 20, 3, 1, p, None) == 2                      # unknown mode
+    assert lib.mi_hbm_stream_ceiling(p, p, 1 << 20, S.STREAM_READ, 0, p, None) == 2
+    assert lib.mi_hbm_stream_ceiling(p, p, 1 << 20, S.STREAM_READ, 9, p, None) == 2
+    assert lib.mi_hbm_stream_ceiling(p, None, 1 << 20, S.STREAM_COPY, 1, p, None) == 2       # a copy needs somewhere to go
+    assert lib.mi_hbm_stream_ceiling(p, p, 1 << 20, S.STREAM_READ, 1, None, None) == 2       # and a read its sink
+    assert lib.mi_hbm_stream_rows_ceiling(None, 1024, 4096, 64, None) == 2
+    assert lib.mi_hbm_stream_rows_ceiling(p, 1024, 4096 + 64, 64, None) == 2                 # rows of whole 128-byte pieces
+    assert lib.mi_hbm_stream_rows_ceiling(p, 1024, 4096, 60, None) == 2                      # eight rows per instruction
+    assert lib.mi_hbm_stream_rows_ceiling(p, 32, 4096, 64, None) == 2                        # more rows per workgroup than rows
+    assert lib.mi_hbm_stream_rows_ceiling(p, 1 << 20, 1 << 16, 1 << 15, None) == 1           # beyond one descriptor's reach
+
+
 def test_static_entry_checks_arguments_and_size_before_touching_the_device():
     """mi_matmul_mfma_static refuses bad modes and operands whose re-packed copies exceed its scratch array before it
     makes any HIP call, so the refusals can be checked without a GPU."""
