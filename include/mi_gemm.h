@@ -266,7 +266,8 @@ int mi_mfma_ceiling(const void* d_operands, size_t operand_bytes, int ab_dtype, 
 
 /* Measurement tool, no reference counterpart: what a kernel that only streams `bytes` of d_src sustains, the yardstick for
  * the GEMM shapes that memory bounds (mi_mfma_ceiling is the one for the shapes the matrix cores bound).
- *   MI_STREAM_READ  16-byte non-temporal vector loads into registers (d_sink: one dword of device memory, keeps them alive);
+ *   MI_STREAM_READ  16-byte non-temporal vector loads into registers (d_sink: one dword of device memory that the kernel
+ *                   scribbles on, to keep the loads alive);
  *   MI_STREAM_DMA   `buffer_load_dwordx4 ... lds`, the GEMM kernel's own producer, into a ring in LDS that is never read:
  *                   72 KB in flight per workgroup, what the 64x128 tile's four-slot ring holds ahead of the slot in use
  *                   (bytes < 4 GiB, workgroups_per_cu <= 2);

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void stream_vector_kernel(const u32x4* __restr
                 __builtin_nontemporal_store(v[u], dst + i + u * stride);
             }
             else {
-                seen |= v[u];
+                seen ^= v[u];
             }
         }
     }
@@ -50,12 +50,12 @@ __global__ __launch_bounds__(256) void stream_vector_kernel(const u32x4* __restr
             __builtin_nontemporal_store(v, dst + i);
         }
         else {
-            seen |= v;
+            seen ^= v;
         }
     }
-    // (keeps the loads alive: a source of all-ones bits is not a benchmark operand)
-    if (!COPY && (seen.x & seen.y & seen.z & seen.w) == 0xffffffffu) {
-        *sink = 1u;
+    // (keeps the loads alive: one lane per workgroup leaves a word that depends on everything the lane has read)
+    if (!COPY && threadIdx.x == 0) {
+        *sink = seen.x ^ seen.y ^ seen.z ^ seen.w;
     }
 }
 

@@ -755,7 +755,7 @@ def test_streaming_probes(gpu):
     for rows_per_wg in (8, 64, 128):
         us = timed_us(lambda: gpu.hbm_stream_rows_ceiling(src.data_ptr(), 4096, 16384, rows_per_wg, st))
         assert n / us * 1e-6 > 1.0, (rows_per_wg, us)
-    assert torch.equal(src, before) and int(sink[0]) == 0
+    assert torch.equal(src, before)
 
 
 @pytest.mark.parametrize("name,dtype", [("f16", 0), ("bf16", 1)])
