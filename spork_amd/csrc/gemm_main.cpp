@@ -11,6 +11,7 @@
 //   gemm --exo M N K [f16|bf16] [style] [param]     one size: the planner and every Exo-named fp32 entry point
 //   gemm --timeline M N K [f16|bf16] [tile code]    in-kernel timeline of one launch
 //   gemm --ceiling  what a register-only MFMA loop sustains on the benchmark's operand values
+//   gemm --calibrate  the planner's two constants per tile, measured on this machine, beside the planner's own
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -53,6 +54,9 @@ int main(int argc, char** argv)
 
     if (argc > 1 && strcmp(argv[1], "--ceiling") == 0) {
         return mfma_ceiling_report({});
+    }
+    if (argc > 1 && strcmp(argv[1], "--calibrate") == 0) {
+        return planner_calibration({});
     }
     if (argc > 1 && strcmp(argv[1], "--timeline") == 0) {
         if (argc < 5) {

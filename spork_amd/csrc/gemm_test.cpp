@@ -531,6 +531,86 @@ int mfma_ceiling_report(gpu_stream_t stream)
     return 0;
 }
 
+// The planner ranks plans by two measured constants per tile: the main-loop time per 64-deep K step with every CU busy, and
+// the cost of a workgroup outside the main loop.  This measures both on the machine at hand, tile by tile, from two
+// one-round problems that differ only in K (bf16 normal data, output stationary, the reference's statistic over 25
+// launches after 30 ms of the same launch), and prints them beside what the planner's own estimate implies for the same two
+// problems: the way to see whether the table still fits a new box or toolchain, and the figures to put into it if not.
+int planner_calibration(gpu_stream_t stream)
+{
+    char name[256], arch[256];
+    int cus = 0;
+    gpu_check(mi_rt_device_info(0, name, arch, &cus, nullptr, nullptr, nullptr), "device info");
+    constexpr uint32_t K1 = 2048, K2 = 6144;
+    printf("one round of each tile on %i CUs, bf16 normal(0,1)/sqrt(K), K = %u and %u\n", cus, K1, K2);
+    printf("%-10s %8s %10s %10s | %12s %12s | %12s %12s\n", "tile", "M x N", "us @K1", "us @K2", "us per K64", "(planner)",
+           "fixed us", "(planner)");
+    void *ev0 = nullptr, *ev1 = nullptr;
+    gpu_check(mi_rt_event_create(&ev0), "event create");
+    gpu_check(mi_rt_event_create(&ev1), "event create");
+    for (int tile = 1; tile < mi_tile_count(); ++tile) {
+        uint32_t bm = 0, bn = 0;
+        int per_cu = 1;
+        gpu_check(mi_tile_shape(tile, &bm, &bn, &per_cu, nullptr), "tile shape");
+        // a grid of tiles that fills every place of one round exactly: 16 x (CUs / 16) tiles, twice that for two per CU
+        if (cus % 16) {
+            continue;
+        }
+        const uint32_t M = bm * 16, N = bn * uint32_t(cus / 16) * uint32_t(per_cu);
+        void* d_a = device_alloc(size_t(2) * M * K2);
+        void* d_b = device_alloc(size_t(2) * N * K2);
+        float* d_c = static_cast<float*>(device_alloc(sizeof(float) * M * N));
+        gpu_check(mi_init_test_data(d_a, M, K2, int(TestDataCode::normal), false, MI_BF16, 1.0 / sqrt(double(K2)), SEED_A, stream), "init");
+        gpu_check(mi_init_test_data(d_b, N, K2, int(TestDataCode::normal), true, MI_BF16, 1.0 / sqrt(double(K2)), SEED_B, stream), "init");
+        double us[2] = {0, 0}, est[2] = {0, 0};
+        bool ok = true;
+        for (int which = 0; which < 2 && ok; ++which) {
+            const uint32_t K = which ? K2 : K1;  // (the same buffers read as M x K and N x K: the values do not matter)
+            const mi_gemm_tensors t{M, N, K, d_a, d_b, d_c, 0, 1, 0, MI_BF16};
+            if (!mi_matmul_mfma_supports(&t, MI_K_OUTPUT_STATIONARY, tile) ||
+                mi_matmul_mfma_estimate_us(&t, MI_K_OUTPUT_STATIONARY, tile, 0, &est[which]) != MI_OK) {
+                ok = false;
+                break;
+            }
+            const int settle = int(30000.0 / std::max(5.0, est[which])) + 1;
+            for (int i = 0; i < settle; ++i) {
+                gpu_check(mi_matmul_mfma(&t, MI_K_OUTPUT_STATIONARY, tile, stream), "matmul");
+                if (i % 32 == 31) {
+                    gpu_check(mi_rt_stream_synchronize(stream), "stream sync");
+                }
+            }
+            float times[25];
+            for (float& ms : times) {
+                gpu_check(mi_rt_event_record(ev0, stream), "event record");
+                gpu_check(mi_matmul_mfma(&t, MI_K_OUTPUT_STATIONARY, tile, stream), "matmul");
+                gpu_check(mi_rt_event_record(ev1, stream), "event record");
+                gpu_check(mi_rt_stream_synchronize(stream), "stream sync");
+                gpu_check(mi_rt_event_elapsed_ms(&ms, ev0, ev1), "elapsed");
+            }
+            std::sort(&times[0], &times[25]);
+            double sum = 0;
+            for (int i = 6; i < 19; ++i) {
+                sum += times[i];  // the middle half (gemm/gemm_test.cu:399-404)
+            }
+            us[which] = sum / 13.0 * 1e3;
+        }
+        if (ok) {
+            const double steps1 = K1 / 64.0, steps2 = K2 / 64.0;
+            const double per_k64 = (us[1] - us[0]) / (steps2 - steps1), fixed = us[0] - steps1 * per_k64;
+            const double est_k64 = (est[1] - est[0]) / (steps2 - steps1), est_fixed = est[0] - steps1 * est_k64;
+            printf("%-10s %4ux%-5u %9.1f %10.1f | %12.3f %12.3f | %12.1f %12.1f\n", mi_tile_name(tile), M, N, us[0], us[1], per_k64,
+                   est_k64, fixed, est_fixed);
+            fflush(stdout);
+        }
+        mi_rt_free(d_a);
+        mi_rt_free(d_b);
+        mi_rt_free(d_c);
+    }
+    mi_rt_event_destroy(ev0);
+    mi_rt_event_destroy(ev1);
+    return 0;
+}
+
 }  // namespace gemm_test_impl
 
 int mfma_ceiling_report(gpu_stream_t stream)
@@ -541,6 +621,11 @@ int mfma_ceiling_report(gpu_stream_t stream)
 int gemm_timeline(TimelineParams params, gpu_stream_t stream)
 {
     return gemm_test_impl::gemm_timeline(params, stream);
+}
+
+int planner_calibration(gpu_stream_t stream)
+{
+    return gemm_test_impl::planner_calibration(stream);
 }
 
 int gemm_test(TestParams params, gpu_stream_t stream)

@@ -139,6 +139,10 @@ struct TimelineParams
 // benchmark's operand distributions and on zeros: the ceiling a GEMM kernel on this power-limited part works under.
 int mfma_ceiling_report(gpu_stream_t stream);
 
+// Measures, tile by tile, the two constants the library's planner prices a tile with (main-loop time per 64-deep K step,
+// per-workgroup cost outside it) and prints them beside what the planner's estimates imply: `gemm --calibrate`.
+int planner_calibration(gpu_stream_t stream);
+
 // Launches the planner's kernel for A MxK, B NxK with in-kernel time stamps and prints, per phase of a workgroup's
 // life (K loop and store issue of each output tile), the min/mean/max duration and the core clock, and per XCD the
 // time its workgroups finish.  Returns non-zero if nothing was recorded.

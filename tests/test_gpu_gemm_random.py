@@ -63,7 +63,13 @@ def _run_case(gpu, case):
             return "needs workspace"
         gpu.matmul_mfma(t, k_mode, tile, H.stream_handle())
     else:
-        gpu.matmul_mfma_ws(t, ws.data_ptr(), size, k_mode, tile, H.stream_handle())
+        # (about half of the cases sum their K partitions or stream-K parts inside the GEMM launch, the rest by a launch
+        # of its own, which is the library's default)
+        was, _ = gpu.matmul_mfma_sum_in_launch((M + N + K // 8) % 2)
+        try:
+            gpu.matmul_mfma_ws(t, ws.data_ptr(), size, k_mode, tile, H.stream_handle())
+        finally:
+            gpu.matmul_mfma_sum_in_launch(was)
     ref = torch.empty((M, N), dtype=torch.float32, device="cuda")
     gpu.matmul_baseline(H.tensors(M, N, K, a, b, ref, dtype, ac, bc, 0), H.stream_handle())
     torch.cuda.synchronize()
