@@ -167,10 +167,11 @@ int mi_matmul_mfma_static(const mi_gemm_tensors* t, int k_mode, int tile, void* 
 /* Where the parts of MI_K_SPLIT_REDUCE and MI_K_STREAM are summed: by a kernel launch of its own behind the GEMM (0, the
  * default), or inside the GEMM launch (1), where the workgroup that stores a tile's last part adds the tile's parts - the
  * reference's scheme (gemm/gemm_sm90.cu:944-963,1004-1095), with plain loads and stores in a fixed order in place of its
- * reduce-adds.  The results are the same bits either way.  The default is the faster way on MI355X on every shape measured
- * (2048 x 2048 x 65536 in four partitions: 404 against 434 us; 160 x 480 x 816 in seven: 7.4 against 21 us): making a part
- * visible to the other XCDs and dropping stale lines takes device-wide cache operations of about 15 us per launch, and only
- * one workgroup per tile sums where the extra launch puts every CU to it.
+ * reduce-adds.  The results are the same bits either way.  The default is the faster way on MI355X on almost every shape
+ * measured (2048 x 2048 x 65536 in four partitions: 412 against 425 us; 160 x 480 x 816 in seven: 7.7 against 12 us; level on
+ * 16384 x 128 x 8192 in two): only one workgroup per tile sums where the extra launch puts every CU to it.  Inside the
+ * launch the parts are stored and read back with device-coherent accesses (`sc1`), so no cache is written back or invalidated
+ * as a whole.  Problems of whole tiles only: a ragged problem sums with the extra launch whatever the setting.
  * The sum inside the launch takes one arrival counter per tile, zero when the launch starts; the counters are an array in
  * the library's own code object (zero when it is loaded, left zero by every launch), dealt out in slabs of 4096 by
  * workspace address: calls that share a workspace are ordered by their caller anyway and share a slab, calls on different

@@ -1283,7 +1283,8 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
         TileDims d;
         tile_dims(plan.tile, c.K, d);
         const uint64_t tiles = (uint64_t)ceil_div(c.M, d.bm) * ceil_div(c.N, d.bn) * c.batches;
-        k.tile_counters = attributes_only ? nullptr : tile_counters_for(workspace_owner ? workspace_owner : workspace, tiles);
+        // (whole tiles only: the range-checked build of the kernel does not carry the sum)
+        k.tile_counters = attributes_only || needs_edge(k, d) ? nullptr : tile_counters_for(workspace_owner ? workspace_owner : workspace, tiles);
         k.c_final = c.c;
         k.ldc_final = c.ldc;
         k.c_final_batch_bytes = c.c_batch_bytes;

@@ -264,6 +264,59 @@ __device__ __forceinline__ void wait_lgkmcnt()
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
 }
 
+// Cache policy of a buffer access (the instruction's aux operand on gfx950): bit 1 `nt`, streaming; bit 4 `sc1`, coherent
+// at device scope - the access is performed where every XCD sees it (a store is written through its XCD's private L2, a
+// load does not take that L2's word for it).  Parts of an output tile that another workgroup, possibly on another XCD,
+// is going to add up inside the same launch are stored and loaded with `sc1`: that is what makes them visible to it
+// without a write-back or an invalidation of a whole L2, which cost about 15 us per launch and hit every workgroup that is
+// still running.
+constexpr int AUX_NT = 2, AUX_NT_SC1 = 2 | 16, AUX_SC1 = 16;
+
+// (Device-only builtins are kept out of lambda bodies, see sched_fence.)
+template <int AUX>
+__device__ __forceinline__ void buffer_store_16B(u32x4 bits, __amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc, voff, soff, AUX);
+}
+template <int AUX>
+__device__ __forceinline__ void buffer_store_4B(uint32_t bits, __amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(bits, rsrc, voff, soff, AUX);
+}
+__device__ __forceinline__ f32x4 load_part(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset, f32x4)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, AUX_SC1));
+}
+__device__ __forceinline__ float load_part(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset, float)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, AUX_SC1));
+}
+
+// A wave's whole tile of 16-wide MFMA tiles with permuted B rows (see TileCfg::perm_row) to global memory: a lane's
+// accumulators of four neighbouring MFMA tiles are four consecutive columns, 16 bytes per store, 256 contiguous bytes per
+// row and instruction.  `voff`: the lane's fixed byte offset; the rest of an address is a scalar.
+template <int AUX, typename Cfg, typename AccT>
+__device__ __forceinline__ void store_wave_tile_16B(const AccT (&acc)[Cfg::MI][Cfg::NI], __amdgpu_buffer_rsrc_t rsrc_c, uint32_t voff,
+                                                    uint32_t ldc)
+{
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+        for (int nq = 0; nq < Cfg::NI / 4; ++nq) {
+#pragma unroll
+            for (int r = 0; r < Cfg::NACC; ++r) {
+                const uint32_t soff = ((mi * Cfg::MT + r) * ldc + nq * 64) * 4u;  // (register r of a 16-wide tile is its row r)
+                const float v0 = acc[mi][4 * nq + 0][r], v1 = acc[mi][4 * nq + 1][r];
+                const float v2 = acc[mi][4 * nq + 2][r], v3 = acc[mi][4 * nq + 3][r];
+                const u32x4 bits = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
+                                    __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
+                buffer_store_16B<AUX>(bits, rsrc_c, voff, soff);
+                after_wide_store();
+            }
+        }
+    }
+}
+
 // Stream-K: the leftover workgroups [j_lo, j_hi) whose runs overlap tail tile t.  Leftover workgroup j owns the
 // leftover (tile, K tile) pairs [j * units / lefts, (j + 1) * units / lefts), units = tiles * kr; tile t's pairs are
 // [t * kr, (t + 1) * kr).  (A run may be empty when there are more leftover workgroups than pairs: see leftover_run_empty.)
@@ -291,14 +344,15 @@ __device__ __forceinline__ bool leftover_run_empty(uint32_t tiles, uint32_t kr, 
     return (uint64_t)j * units / lefts == (uint64_t)(j + 1) * units / lefts;
 }
 
-// A workgroup has stored one part of an output tile: make the part visible to the whole device, count it, and tell
-// every thread of the workgroup whether it was the tile's last part (the counter is then set back to zero, for the next
-// launch: nobody else touches it any more in this one).  Nobody waits for anybody.  `lds_flag`: a dword of LDS that no one
-// is using.  The device-scope release writes this XCD's L2 back (the XCDs' L2s are private), the acquire drops what this
-// one may hold of the other parts' addresses from an earlier launch.
+// A workgroup has stored one part of an output tile (with device-coherent stores, AUX_NT_SC1): count it, and tell every
+// thread of the workgroup whether it was the tile's last part (the counter is then set back to zero, for the next launch:
+// nobody else touches it any more in this one).  Nobody waits for anybody.  `lds_flag`: a dword of LDS that no one is
+// using.  Every wave waits until its own stores have been performed (vmcnt counts a store until the level that holds it
+// coherently has it), the barrier gathers the waves, and only then is the arrival counted, by a device-scope atomic;
+// whoever reads the count as complete reads the parts with device-coherent loads (load_part), which go past the L2.
 __device__ __forceinline__ bool part_stored_is_it_the_last(uint32_t* counter, uint32_t expected, volatile lds_u32* lds_flag)
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -309,24 +363,22 @@ __device__ __forceinline__ bool part_stored_is_it_the_last(uint32_t* counter, ui
         *lds_flag = last ? 1u : 0u;
     }
     __syncthreads();
-    const bool last = *lds_flag != 0u;
-    if (last) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    }
-    return last;
+    return *lds_flag != 0u;
 }
 
 // C tile = part(0) + part(1) + ... + part(n_parts - 1), added in that order (so the result does not depend on which
 // workgroup does the adding, or when).  part(i) is where element (0, 0) of the tile lies in part i; every part has row
-// pitch `ld_part`.  T = f32x4: every pointer and pitch is a multiple of 16 bytes and columns come four at a time; T =
-// float otherwise.  Rows from `m_rem` and columns from `n_rem` on do not exist.  All parts of U places of a thread are
-// requested before the first is awaited (up to four parts at a time): a lone workgroup has only its own loads in flight
-// to cover the memory latency with.  (U = 8 takes about 160 vector registers.)
-template <int BM, int BN, int NTHREADS, typename T, uint32_t U, typename PartFn>
+// pitch `ld_part` (the tile's last element less than 2 GiB from its first).  T = f32x4: every pointer and pitch is a
+// multiple of 16 bytes and columns come four at a time; T = float otherwise.  Rows from `m_rem` and columns from `n_rem` on
+// do not exist.  The parts of U places of a thread, G parts at a time, are requested before the first is awaited: a lone
+// workgroup has only its own loads in flight to cover the memory latency with (these loads go past the L2).  U * (G + 1)
+// values of T are live at once.
+template <int BM, int BN, int NTHREADS, typename T, uint32_t U, uint32_t G, typename PartFn>
 __device__ __forceinline__ void sum_tile_parts(PartFn part, uint32_t n_parts, uint32_t ld_part, float* c_tile, uint32_t ldc,
                                                int32_t m_rem, int32_t n_rem)
 {
     constexpr uint32_t W = sizeof(T) / 4, Q = BN / W, TOTAL = BM * Q;
+    constexpr uint32_t REACH = 0x80000000u;  // bytes a part's descriptor covers (offsets beyond it would read as zero)
     for (uint32_t first = threadIdx.x; first < TOTAL; first += NTHREADS * U) {
         uint32_t at_part[U], at_c[U];
         bool exists[U];
@@ -335,48 +387,38 @@ __device__ __forceinline__ void sum_tile_parts(PartFn part, uint32_t n_parts, ui
             const uint32_t idx = first + u * NTHREADS, row = idx / Q, col = (idx % Q) * W;
             exists[u] = idx < TOTAL && (int32_t)row < m_rem && (int32_t)col < n_rem;
             // (a place that does not exist reads element (0, 0), which does, and stores nothing)
-            at_part[u] = exists[u] ? row * ld_part + col : 0u;
+            at_part[u] = exists[u] ? (row * ld_part + col) * 4u : 0u;
             at_c[u] = row * ldc + col;
         }
         T acc[U];
-        const float* const p0 = part(0);
-#pragma unroll
-        for (uint32_t u = 0; u < U; ++u) {
-            acc[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(p0 + at_part[u]));
-        }
-        uint32_t i = 1;
-        for (; i + 2 < n_parts; i += 3) {
-            const float* const q0 = part(i), * const q1 = part(i + 1), * const q2 = part(i + 2);
-            T v0[U], v1[U], v2[U];
+        {
+            const __amdgpu_buffer_rsrc_t r0 = make_rsrc(part(0), REACH);
 #pragma unroll
             for (uint32_t u = 0; u < U; ++u) {
-                v0[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
-                v1[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q1 + at_part[u]));
-                v2[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q2 + at_part[u]));
-            }
-#pragma unroll
-            for (uint32_t u = 0; u < U; ++u) {
-                acc[u] = ((acc[u] + v0[u]) + v1[u]) + v2[u];
+                acc[u] = load_part(r0, at_part[u], T{});
             }
         }
-        if (i + 1 < n_parts) {
-            const float* const q0 = part(i), * const q1 = part(i + 1);
-            T v0[U], v1[U];
+        for (uint32_t i = 1; i < n_parts; i += G) {
+            // up to G parts at once; a part beyond the last is not loaded and not added (the adds stay in part order)
+            T v[G][U];
 #pragma unroll
-            for (uint32_t u = 0; u < U; ++u) {
-                v0[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
-                v1[u] = __builtin_nontemporal_load(reinterpret_cast<const T*>(q1 + at_part[u]));
+            for (uint32_t k = 0; k < G; ++k) {
+                if (i + k < n_parts) {
+                    const __amdgpu_buffer_rsrc_t rk = make_rsrc(part(i + k), REACH);
+#pragma unroll
+                    for (uint32_t u = 0; u < U; ++u) {
+                        v[k][u] = load_part(rk, at_part[u], T{});
+                    }
+                }
             }
 #pragma unroll
-            for (uint32_t u = 0; u < U; ++u) {
-                acc[u] = (acc[u] + v0[u]) + v1[u];
-            }
-        }
-        else if (i < n_parts) {
-            const float* const q0 = part(i);
+            for (uint32_t k = 0; k < G; ++k) {
+                if (i + k < n_parts) {
 #pragma unroll
-            for (uint32_t u = 0; u < U; ++u) {
-                acc[u] += __builtin_nontemporal_load(reinterpret_cast<const T*>(q0 + at_part[u]));
+                    for (uint32_t u = 0; u < U; ++u) {
+                        acc[u] += v[k][u];
+                    }
+                }
             }
         }
 #pragma unroll
@@ -1194,27 +1236,18 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             // MT = 32: one dword per lane, two full 128 B row segments per instruction.  MT = 16: four MFMA tiles at a
             // time, 16 B per lane, four 256 B row segments per instruction (see PERM).  Non-temporal, so C does not
             // displace the A/B panels that other tiles are re-reading from the L2.
-            constexpr int NT = 2;
+            constexpr int NT = AUX_NT;
             if constexpr (!EDGE) {
                 const __amdgpu_buffer_rsrc_t rsrc_c =
                     make_rsrc(c_wave, ((Cfg::TM - 1) * p.ldc + Cfg::TN) * 4u);
                 const uint32_t voff = (4u * g * p.ldc + Cfg::template acc_col<PERM>(0, lrc)) * 4u;
                 if constexpr (PERM) {
-#pragma unroll
-                    for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-                        for (int nq = 0; nq < NI / 4; ++nq) {
-#pragma unroll
-                            for (int r = 0; r < NACC; ++r) {
-                                const uint32_t soff = ((mi * MT + row_of(r)) * p.ldc + nq * 64) * 4u;
-                                const float v0 = acc[mi][4 * nq + 0][r], v1 = acc[mi][4 * nq + 1][r];
-                                const float v2 = acc[mi][4 * nq + 2][r], v3 = acc[mi][4 * nq + 3][r];
-                                const u32x4 bits = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
-                                                    __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
-                                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_c, voff, soff, NT);
-                                after_wide_store();
-                            }
-                        }
+                    // (a part that another workgroup will add up inside this launch is stored device-coherently as well)
+                    if (p.tile_counters != nullptr) {
+                        store_wave_tile_16B<AUX_NT_SC1, Cfg>(acc, rsrc_c, voff, p.ldc);
+                    }
+                    else {
+                        store_wave_tile_16B<AUX_NT, Cfg>(acc, rsrc_c, voff, p.ldc);
                     }
                 }
                 else {
@@ -1226,7 +1259,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                             for (int r = 0; r < NACC; ++r) {
                                 const uint32_t soff = ((mi * MT + row_of(r)) * p.ldc + ni * MT) * 4u;
                                 const float v = acc[mi][ni][r];  // (bit_cast straight from a vector element reads element 0)
-                                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc_c, voff, soff, NT);
+                                buffer_store_4B<NT>(__builtin_bit_cast(uint32_t, v), rsrc_c, voff, soff);
                             }
                         }
                     }
@@ -1255,7 +1288,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                                     const float v2 = acc[mi][4 * nq + 2][r], v3 = acc[mi][4 * nq + 3][r];
                                     const u32x4 bits = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
                                                         __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
-                                    __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_c, inside ? voff + soff : OOB, 0u, NT);
+                                    buffer_store_16B<NT>(bits, rsrc_c, inside ? voff + soff : OOB, 0u);
                                     after_wide_store();
                                 }
                             }
@@ -1274,8 +1307,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                                 const uint32_t soff = ((uint32_t)row * p.ldc + col) * 4u;
                                 const bool inside = row < m_left && (int32_t)col < n_left;
                                 const float v = acc[mi][ni][r];
-                                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc_c,
-                                                                      inside ? voff + soff : OOB, 0u, NT);
+                                buffer_store_4B<NT>(__builtin_bit_cast(uint32_t, v), rsrc_c, inside ? voff + soff : OOB, 0u);
                             }
                         }
                     }
@@ -1283,7 +1315,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
             }
         }
 
-        if constexpr (!ATOMIC) {
+        if constexpr (!ATOMIC && !EDGE) {
             if (p.tile_counters != nullptr) {
                 // This was one part of its tile (a K partition's copy, or a stream-K part).  Whoever stores a tile's last
                 // part adds them all up, in their fixed order, into the caller's C.
@@ -1318,10 +1350,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                         };
                         const bool vec = p.ldc_final % 4u == 0 && ((uintptr_t)cur.final_tile & 15u) == 0;
                         if (vec) {
-                            sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
+                            sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U, 3>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
                         }
                         else {
-                            sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
+                            sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4, 3>(part, S + left_parts, BN, cur.final_tile, p.ldc_final, BM, BN);
                         }
                     }
                 }
@@ -1331,10 +1363,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(const GemmArgs p
                     const bool vec = p.ldc % 4u == 0 && p.ldc_final % 4u == 0 && p.c_split_bytes % 16u == 0 &&
                                      (((uintptr_t)part0 | (uintptr_t)cur.final_tile) & 15u) == 0;
                     if (vec) {
-                        sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
+                        sum_tile_parts<BM, BN, Cfg::NTHREADS, f32x4, SUM_U, 3>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
                     }
                     else {
-                        sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
+                        sum_tile_parts<BM, BN, Cfg::NTHREADS, float, 4, 3>(part, cur.parts, p.ldc, cur.final_tile, p.ldc_final, cur.m_rem, cur.n_rem);
                     }
                 }
             }

@@ -153,8 +153,9 @@ int launch_cfg(const Canonical& c, uint32_t k_splits, bool edge, hipStream_t str
     args.b_batch_bytes = c.b_batch_bytes;
     args.c_batch_bytes = c.c_batch_bytes;
     args.c_split_bytes = k_splits > 1 ? c.c_split_bytes : 0;
-    // (K partitions' copies of C, or stream-K parts; a sum inside the launch needs one or the other)
-    const bool sums_inside = c.tile_counters != nullptr && c.c_final != nullptr && (args.c_split_bytes != 0 || c.stream_k_workgroups > 0);
+    // (K partitions' copies of C, or stream-K parts; a sum inside the launch needs one or the other, and whole tiles: the
+    // range-checked build does not carry it, see run_mfma)
+    const bool sums_inside = c.tile_counters != nullptr && c.c_final != nullptr && !edge && (args.c_split_bytes != 0 || c.stream_k_workgroups > 0);
     args.tile_counters = sums_inside ? c.tile_counters : nullptr;
     args.c_final = c.c_final;
     args.ldc_final = c.ldc_final ? c.ldc_final : c.N;
