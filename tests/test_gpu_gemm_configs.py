@@ -86,6 +86,45 @@ def test_config_sampled_oracle_freivalds_and_device_baseline(gpu, oracle, name):
     assert dev < TOL
 
 
+def test_deep_k_config_as_benchmarked_with_the_preferred_workspace(gpu, oracle):
+    """C5 the way the benchmark runs it: with the workspace the planner prefers, which makes it four K partitions of
+    256x256 tiles summed from copies of C.  Checked against the oracle on sampled rows and against the device baseline
+    over the whole matrix; summed by a launch of its own and inside the GEMM launch the bits must be the same; stream-K
+    with the same room must be as accurate."""
+    M, N, K, dtype, a, b = _inputs("c5")
+    c = H.poisoned_c(M, N)
+    t = H.tensors(M, N, K, a, b, c, dtype)
+    _, pref = gpu.matmul_mfma_workspace_bytes_for(t)
+    ws = torch.empty(pref, dtype=torch.uint8, device="cuda")
+    plan = gpu.matmul_mfma_describe(t, workspace_bytes=pref)
+    assert "split k (workspace sum)" in plan, plan
+    results = []
+    for in_launch in (False, True):
+        c.view(torch.uint8).fill_(0x7D)
+        ws.fill_(0xFF)
+        was, _ = gpu.matmul_mfma_sum_in_launch(in_launch)
+        try:
+            gpu.matmul_mfma_ws(t, ws.data_ptr(), pref, gpu.K_AUTO, gpu.TILE_AUTO, H.stream_handle())
+        finally:
+            gpu.matmul_mfma_sum_in_launch(was)
+        torch.cuda.synchronize()
+        results.append(c.clone())
+    assert torch.equal(results[0], results[1])
+    ha, hb = H.to_host_u16(a), H.to_host_u16(b)
+    rng = np.random.default_rng(11)
+    edges = np.arange(0, M, 256)
+    rows = np.unique(np.concatenate([edges, edges + 255, rng.integers(0, M, 16)]))[:32]
+    ref_rows = oracle.gemm_f64_rows(M, N, K, ha, hb, dtype, rows)
+    err_rows = np.abs(results[0][rows].cpu().numpy().astype(np.float64) - ref_rows).max() / np.abs(ref_rows).max()
+    dev = _device_baseline_rel_err(gpu, M, N, K, a, b, results[0], dtype)
+    c.view(torch.uint8).fill_(0x7D)
+    gpu.matmul_mfma_ws(t, ws.data_ptr(), pref, gpu.K_STREAM, gpu.TILE_AUTO, H.stream_handle())
+    torch.cuda.synchronize()
+    dev_stream = _device_baseline_rel_err(gpu, M, N, K, a, b, c, dtype)
+    print(plan, "rows", err_rows, "device baseline", dev, "stream-K", dev_stream)
+    assert err_rows < TOL and dev < TOL and dev_stream < TOL
+
+
 def test_headline_known_answer_tiled_times_identity(gpu, oracle):
     """gemm/gemm_main.cpp:81-85 at the headline size: C must reproduce A exactly."""
     M = N = K = 8192
