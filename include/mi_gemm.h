@@ -310,6 +310,17 @@ int mi_tile_count(void);
 const char* mi_tile_name(int tile);
 int mi_tile_shape(int tile, uint32_t* out_bm, uint32_t* out_bn, int* out_workgroups_per_cu, int* out_has_32_deep_twin);
 const char* mi_k_mode_name(int k_mode);
+/* The two constants MI_K_AUTO prices a tile with: microseconds per 64-deep K step of one round of workgroups, and
+ * microseconds per workgroup besides its K loop (ring fill, stores, dispatch).  They were measured on MI355X; on another
+ * board, power limit or ROCm release `gemm --calibrate` measures them again in a minute and prints them beside these and
+ * as one line for the environment variable MI_GEMM_PLANNER_CONSTANTS ("256x256=1.26/16.1,64x128=0.31/5.4", read when
+ * the library is loaded).  mi_tile_set_planner_constants replaces a tile's pair for the rest of the process (the figures
+ * derived from it - a lone workgroup of a tile that shares its CU, short launches - are scaled with it); it is not
+ * synchronised with calls that are planning at the same time, so set the constants before the first GEMM call.  No
+ * counterpart in the reference, whose schedule is chosen by the caller (gemm/gemm_sm90.h:5-12).
+ * MI_ERR_BAD_ARGUMENT: unknown tile, or a constant that is not in (0, 1000]. */
+int mi_tile_planner_constants(int tile, double* out_us_per_k64, double* out_fixed_us);
+int mi_tile_set_planner_constants(int tile, double us_per_k64, double fixed_us);
 
 /* ------------------------------------------------------------------------------- harness device helpers */
 /* Test-data styles; 0..2 replace `enum class TestDataCode` (gemm/gemm_test.h:6-11); 3,4 are the seeded

@@ -140,6 +140,8 @@ def lib() -> C.CDLL:
     sig("mi_tile_name", C.c_char_p, [i32])
     sig("mi_tile_count", i32, [])
     sig("mi_tile_shape", i32, [i32, C.POINTER(u32), C.POINTER(u32), ip, ip])
+    sig("mi_tile_planner_constants", i32, [i32, C.POINTER(C.c_double), C.POINTER(C.c_double)])
+    sig("mi_tile_set_planner_constants", i32, [i32, C.c_double, C.c_double])
     sig("mi_matmul_mfma_prepare", i32, [tp, i32, i32, sz])
     sig("mi_matmul_mfma_sum_in_launch", i32, [i32, C.POINTER(C.c_uint64)])
     sig("mi_k_mode_name", C.c_char_p, [i32])
@@ -225,6 +227,18 @@ def tile_shape(tile: int) -> dict:
     check(lib().mi_tile_shape(tile, C.byref(bm), C.byref(bn), C.byref(per_cu), C.byref(twin)), "mi_tile_shape")
     return {"code": tile, "name": lib().mi_tile_name(tile).decode(), "bm": bm.value, "bn": bn.value,
             "workgroups_per_cu": per_cu.value, "has_32_deep_twin": bool(twin.value)}
+
+
+def tile_planner_constants(tile: int) -> tuple:
+    """(microseconds per 64-deep K step of a round, microseconds per workgroup besides its K loop) the planner prices `tile` with."""
+    k64, fixed = C.c_double(), C.c_double()
+    check(lib().mi_tile_planner_constants(tile, C.byref(k64), C.byref(fixed)), "mi_tile_planner_constants")
+    return k64.value, fixed.value
+
+
+def tile_set_planner_constants(tile: int, us_per_k64: float, fixed_us: float) -> None:
+    """Replaces the pair for the rest of the process (what `gemm --calibrate` measures on the machine at hand)."""
+    check(lib().mi_tile_set_planner_constants(tile, us_per_k64, fixed_us), "mi_tile_set_planner_constants")
 
 
 def tiles() -> list:

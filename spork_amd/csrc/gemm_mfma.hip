@@ -3,7 +3,10 @@
 // gemm/gemm_sm90.cu:1200-1360).
 #include "gemm_mfma_launch.hpp"
 
+#include <atomic>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
 
 namespace mi_gemm {
@@ -28,10 +31,13 @@ MI_TILE_TWINS(MI_GEMM_DECLARE_CFG)
             alone_k64,                                                                                      \
             alone_us,                                                                                       \
             max_k},
-static const TileRow TILES[] = {MI_TILE_TABLE(MI_ROW_ENTRY)};
+// (not const: the two leading planner constants of a row can be replaced at run time, see mi_tile_set_planner_constants)
+static TileRow TILES[] = {MI_TILE_TABLE(MI_ROW_ENTRY)};
 #undef MI_ROW_ENTRY
 constexpr int TILE_ROWS = sizeof(TILES) / sizeof(TILES[0]);
 static_assert(TILE_ROWS == MI_TILE_COUNT_ - 1, "one table row per tile code of the ABI");
+// Counts the replacements of planner constants, so that answers remembered under older ones are not given again.
+static std::atomic<uint32_t> planner_constants_generation{0};
 
 // The row of a tile code, or null (MI_TILE_AUTO and unknown codes have none).
 static const TileRow* tile_row(int tile)
@@ -427,6 +433,7 @@ static bool make_plan(const Canonical& c, int k_mode, int tile, size_t partial_s
         uint32_t c_low_bits;
         int k_mode, tile, cus;
         size_t partial_space;
+        uint32_t constants;  // (planner_constants_generation when the answer was found)
         bool valid, found;
         Plan plan;
     };
@@ -435,11 +442,12 @@ static bool make_plan(const Canonical& c, int k_mode, int tile, size_t partial_s
     static thread_local int next_memo = 0;
     const uint32_t c_low_bits = (uint32_t)((uintptr_t)c.c % 16);
     const uint32_t ab_low_bits = (uint32_t)(((uintptr_t)c.a | (uintptr_t)c.b) % 128);
+    const uint32_t generation = planner_constants_generation.load(std::memory_order_relaxed);
     for (const Memo& memo : memos) {
         if (memo.valid && memo.M == c.M && memo.N == c.N && memo.K == c.K && memo.batches == c.batches &&
             memo.c_batch_bytes == c.c_batch_bytes && memo.lda == c.lda && memo.ldb == c.ldb && memo.ab_low_bits == ab_low_bits &&
             memo.c_low_bits == c_low_bits && memo.k_mode == k_mode &&
-            memo.tile == tile && memo.cus == cus && memo.partial_space == partial_space) {
+            memo.tile == tile && memo.cus == cus && memo.partial_space == partial_space && memo.constants == generation) {
             plan = memo.plan;
             return memo.found;
         }
@@ -447,7 +455,7 @@ static bool make_plan(const Canonical& c, int k_mode, int tile, size_t partial_s
     plan = Plan{MI_TILE_AUTO, MI_K_OUTPUT_STATIONARY, 1, 0, 0.0};
     const bool found = search_plan(c, k_mode, tile, partial_space, cus, plan);
     memos[next_memo] = {c.M,        c.N,    c.K,  c.batches, c.c_batch_bytes, c.lda, c.ldb, ab_low_bits,
-                        c_low_bits, k_mode, tile, cus,       partial_space,   true,  found, plan};
+                        c_low_bits, k_mode, tile, cus,       partial_space,   generation, true,  found, plan};
     next_memo = (next_memo + 1) % MEMOS;
     return found;
 }
@@ -1315,6 +1323,39 @@ static int run_mfma(const mi_gemm_tensors* t, int k_mode, int tile, void* worksp
 
 using namespace mi_gemm;
 
+// MI_GEMM_PLANNER_CONSTANTS="256x256=1.26/16.1,64x128=0.31/5.4": the line `gemm --calibrate` prints for the machine at
+// hand, applied when the library is loaded.  Entries that do not parse or name no tile are reported and skipped.
+static int apply_planner_environment()
+{
+    const char* const text = std::getenv("MI_GEMM_PLANNER_CONSTANTS");
+    if (text == nullptr) {
+        return 0;
+    }
+    int applied = 0;
+    for (const char* at = text; *at != 0;) {
+        const char* end = std::strchr(at, ',');
+        end = end ? end : at + std::strlen(at);
+        char name[32];
+        double k64 = 0, fixed = 0;
+        int used = 0;
+        bool ok = false;
+        if (std::sscanf(at, " %31[0-9x]=%lf/%lf %n", name, &k64, &fixed, &used) == 3 && at + used == end) {
+            for (int tile = 1; tile <= TILE_ROWS && !ok; ++tile) {
+                ok = std::strcmp(TILES[tile - 1].name, name) == 0 && mi_tile_set_planner_constants(tile, k64, fixed) == MI_OK;
+            }
+        }
+        if (ok) {
+            ++applied;
+        }
+        else {
+            std::fprintf(stderr, "mi_gemm: MI_GEMM_PLANNER_CONSTANTS: skipped '%.*s'\n", (int)(end - at), at);
+        }
+        at = *end ? end + 1 : end;
+    }
+    return applied;
+}
+static const int planner_environment_applied = apply_planner_environment();
+
 extern "C" {
 
 int mi_matmul_mfma_plan(const mi_gemm_tensors* t, int k_mode, int tile, int* out_tile, int* out_k_mode, int* out_k_splits)
@@ -1865,6 +1906,44 @@ int mi_tile_shape(int tile, uint32_t* out_bm, uint32_t* out_bn, int* out_workgro
     if (out_has_32_deep_twin) {
         *out_has_32_deep_twin = row->twin[0] != nullptr ? 1 : 0;
     }
+    return MI_OK;
+}
+
+int mi_tile_planner_constants(int tile, double* out_us_per_k64, double* out_fixed_us)
+{
+    const TileRow* const row = tile_row(tile);
+    if (row == nullptr) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    if (out_us_per_k64) {
+        *out_us_per_k64 = row->us_k64;
+    }
+    if (out_fixed_us) {
+        *out_fixed_us = row->fixed_us;
+    }
+    return MI_OK;
+}
+
+int mi_tile_set_planner_constants(int tile, double us_per_k64, double fixed_us)
+{
+    if (tile_row(tile) == nullptr || !(us_per_k64 > 0.0) || !(fixed_us > 0.0) || us_per_k64 > 1e3 || fixed_us > 1e3) {
+        return MI_ERR_BAD_ARGUMENT;
+    }
+    TileRow& row = TILES[tile - 1];
+    // a tile that has a CU to itself has one pair of constants; the tile that shares a CU keeps its figures for a
+    // workgroup running alone, scaled as the pair's are
+    if (row.per_cu == 1) {
+        row.alone_k64 = us_per_k64;
+        row.alone_us = fixed_us;
+    }
+    else {
+        row.alone_k64 *= us_per_k64 / row.us_k64;
+        row.alone_us *= fixed_us / row.fixed_us;
+    }
+    row.short_us *= fixed_us / row.fixed_us;
+    row.us_k64 = us_per_k64;
+    row.fixed_us = fixed_us;
+    planner_constants_generation.fetch_add(1, std::memory_order_relaxed);
     return MI_OK;
 }
 

@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <string>
 #include <vector>
 
 namespace gemm_test_impl {
@@ -548,6 +549,7 @@ int planner_calibration(gpu_stream_t stream)
     void *ev0 = nullptr, *ev1 = nullptr;
     gpu_check(mi_rt_event_create(&ev0), "event create");
     gpu_check(mi_rt_event_create(&ev1), "event create");
+    std::string environment;
     for (int tile = 1; tile < mi_tile_count(); ++tile) {
         uint32_t bm = 0, bn = 0;
         int per_cu = 1;
@@ -601,6 +603,11 @@ int planner_calibration(gpu_stream_t stream)
             printf("%-10s %4ux%-5u %9.1f %10.1f | %12.3f %12.3f | %12.1f %12.1f\n", mi_tile_name(tile), M, N, us[0], us[1], per_k64,
                    est_k64, fixed, est_fixed);
             fflush(stdout);
+            if (per_k64 > 0 && fixed > 0) {
+                char entry[64];
+                snprintf(entry, sizeof(entry), "%s%s=%.3f/%.1f", environment.empty() ? "" : ",", mi_tile_name(tile), per_k64, fixed);
+                environment += entry;
+            }
         }
         mi_rt_free(d_a);
         mi_rt_free(d_b);
@@ -608,6 +615,8 @@ int planner_calibration(gpu_stream_t stream)
     }
     mi_rt_event_destroy(ev0);
     mi_rt_event_destroy(ev1);
+    // (what the library reads when it is loaded; mi_tile_set_planner_constants does the same from code)
+    printf("to plan with the measured figures:\nMI_GEMM_PLANNER_CONSTANTS=%s\n", environment.c_str());
     return 0;
 }
 

@@ -5,6 +5,7 @@ import ctypes as C
 import os
 import re
 import subprocess
+import sys
 
 import pytest
 
@@ -460,6 +461,49 @@ def test_planner_picks_for_the_benchmark_configurations():
     assert (p["tile"], p["k_splits"]) == ("128x128", 1)
     with pytest.raises(S.MiGemmError):
         S.matmul_mfma_plan(_t(100, 100, 100))
+
+
+def test_planner_constants_can_be_replaced_and_read_from_the_environment():
+    """The planner's two constants per tile are data: readable, replaceable for the process (what `gemm --calibrate`
+    measures goes in here), and taken from MI_GEMM_PLANNER_CONSTANTS when the library is loaded.  The estimate of a
+    forced plan follows them; bad values and unknown tiles are refused; a child process shows the environment path."""
+    lib = S.lib()
+    tile = S.TILE_256x256
+    k64, fixed = S.tile_planner_constants(tile)
+    assert 0.5 < k64 < 3.0 and 5.0 < fixed < 40.0
+    t = _t(8192, 8192, 8192, S.BF16)
+    before = S.matmul_mfma_estimate_us(t, S.K_OUTPUT_STATIONARY, tile)
+    try:
+        S.tile_set_planner_constants(tile, 2.0 * k64, fixed)
+        assert S.tile_planner_constants(tile) == (2.0 * k64, fixed)
+        assert S.matmul_mfma_estimate_us(t, S.K_OUTPUT_STATIONARY, tile) > 1.8 * before - 100.0
+        # the planner now prefers another tile for the same problem
+        assert S.matmul_mfma_plan(t)["tile"] != "256x256"
+    finally:
+        S.tile_set_planner_constants(tile, k64, fixed)
+    assert S.matmul_mfma_estimate_us(t, S.K_OUTPUT_STATIONARY, tile) == pytest.approx(before)
+    assert S.matmul_mfma_plan(t)["tile"] == "256x256"
+    # the tile that shares its CU: the figures of a lone workgroup scale with the pair's and come back
+    two = next(x["code"] for x in S.tiles() if x["workgroups_per_cu"] == 2)
+    k2, f2 = S.tile_planner_constants(two)
+    small = _t(192, 128, 1024)
+    lone = S.matmul_mfma_estimate_us(small, S.K_OUTPUT_STATIONARY, two)
+    try:
+        S.tile_set_planner_constants(two, 2.0 * k2, 2.0 * f2)
+        assert S.matmul_mfma_estimate_us(small, S.K_OUTPUT_STATIONARY, two) == pytest.approx(2.0 * lone, rel=0.02)
+    finally:
+        S.tile_set_planner_constants(two, k2, f2)
+    assert S.matmul_mfma_estimate_us(small, S.K_OUTPUT_STATIONARY, two) == pytest.approx(lone)
+    for bad in ((0, 1.0, 1.0), (S.tile_count(), 1.0, 1.0), (tile, 0.0, 1.0), (tile, 1.0, -1.0), (tile, float("nan"), 1.0),
+                (tile, 1.0, 1e4)):
+        assert lib.mi_tile_set_planner_constants(*bad) == 2
+    assert lib.mi_tile_planner_constants(0, None, None) == 2 and lib.mi_tile_planner_constants(tile, None, None) == 0
+    code = ("import spork_amd as S; print(S.tile_planner_constants(S.TILE_256x256), S.tile_planner_constants(S.TILE_64x128), "
+            "S.tile_planner_constants(S.TILE_128x128))")
+    env = dict(os.environ, MI_GEMM_PLANNER_CONSTANTS="256x256=1.5/20.5, 64x128=0.3/5,7x7=1/1,128x128=oops")
+    out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, check=True)
+    assert out.stdout.strip() == f"(1.5, 20.5) (0.3, 5.0) {S.tile_planner_constants(S.TILE_128x128)}", out.stdout
+    assert "skipped '7x7=1/1'" in out.stderr and "skipped '128x128=oops'" in out.stderr
 
 
 def test_host_driver_is_built_against_the_abi_only():
